@@ -1,0 +1,181 @@
+/*
+ * libvlgpu - C ABI of the MI355X (gfx950) kernels behind the vectorlink_gpu
+ * Python surface: gathered cosine distances, batched sorted queues, candidate
+ * dedup / exclusion, the beam-search loop, detour pruning and exact kNN tiles.
+ *
+ * The reference has no FFI of its own: its boundary is the set of Python
+ * launcher functions in vectorlink_gpu/kernels.py plus the Queue class, all
+ * taking torch tensors.  Each entry point below names the launcher or method
+ * it stands in for (paths relative to the reference checkout).
+ *
+ * Conventions
+ *  - every pointer is a DEVICE pointer unless its name starts with host_;
+ *  - matrices are row-major and dense unless a *_stride argument (in
+ *    elements) is given; sizes are int64_t;
+ *  - ids are int32 with VL_MAXINT as the empty id, distances are float32 with
+ *    VL_MAXFLOAT as the empty distance (vectorlink_gpu/constants.py:5-6);
+ *    real ids must be below 2^30 (bit 30 is the reference's duplicate flag,
+ *    kernels.py:325);
+ *  - `stream` is a hipStream_t passed as void*; work is enqueued on it and
+ *    the call returns without synchronising unless stated otherwise;
+ *  - the library allocates no device memory: scratch comes from the caller
+ *    as a workspace whose size the matching *_workspace_bytes call reports;
+ *  - return value 0 is success; a negative value is an error whose text
+ *    vl_last_error() returns (thread local).  Shapes are validated on the
+ *    host before anything is launched.
+ */
+#ifndef VLGPU_H
+#define VLGPU_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VL_MAXINT 2147483647
+#define VL_MAXFLOAT 3.4028e37f
+#define VL_DUP_FLAG (1 << 30)
+
+#define VL_OK 0
+#define VL_ERR_ARG (-1)      /* bad shape / null pointer / unsupported size */
+#define VL_ERR_HIP (-2)      /* a HIP runtime call failed */
+#define VL_ERR_WORKSPACE (-3) /* workspace too small */
+
+const char *vl_last_error(void);
+int vl_version(void);
+
+/* ---- distances -------------------------------------------------------- */
+
+/* out[r, j] = clamp((1 - <queries[r], vectors[ids[r, j]]>) / 2, 0, 1);
+ * VL_MAXFLOAT where ids[r, j] is VL_MAXINT or outside [0, n_vectors).
+ * With queries == vectors and ids == beams this is calculate_distances
+ * (kernels.py:174-201, kernel 130-171); with circulant seed ids it is the
+ * seed-distance step of initial_search_queue (ann.py:228-229). */
+int vl_gather_distances(const float *queries, int64_t n_rows,
+                        const float *vectors, int64_t n_vectors, int64_t dim,
+                        const int32_t *ids, int64_t width,
+                        float *out, void *stream);
+
+/* search_from_seeds (kernels.py:260-311, kernel 204-257): for row b, visit
+ * slot s, neighbour slot k: nb = beams[visit[b,s], k];
+ * idx_out[b, s*width+k] = nb, dist_out[...] = d(vectors[nb], queries[b]).
+ * A VL_MAXINT visit id or neighbour id yields (VL_MAXINT, VL_MAXFLOAT). */
+int vl_search_from_seeds(const float *queries, int64_t n_rows, int64_t dim,
+                         const int32_t *visit, int64_t n_visit,
+                         const int32_t *beams, int64_t n_nodes, int64_t width,
+                         const float *vectors, int64_t n_vectors,
+                         int32_t *idx_out, float *dist_out, void *stream);
+
+/* ---- seed graphs ------------------------------------------------------ */
+
+/* generate_circulant_beams / generate_queue_circulants (utils.py:26-41):
+ * out[r, k] = sort_k(row0 + r + primes[k]) % modulus. primes: device int32. */
+int vl_circulants(int32_t *out, int64_t rows, int64_t row0, int64_t modulus,
+                  const int32_t *primes, int64_t n_primes, void *stream);
+
+/* ---- dedup / exclusion / gather helpers ------------------------------- */
+
+/* dedup_tensor_ (kernels.py:370-380): per row, a slot whose id equals its
+ * left neighbour's (bit 30 ignored) becomes VL_MAXINT.  In place. */
+int vl_dedup_ids(int32_t *ids, int64_t rows, int64_t cols, void *stream);
+
+/* dedup_tensor_pair_ (kernels.py:383-397): same, and the distance of a
+ * punched slot becomes VL_MAXFLOAT.  In place. */
+int vl_dedup_pairs(int32_t *ids, float *dists, int64_t rows, int64_t cols, void *stream);
+
+/* punchout_excluded_ (kernels.py:491-501): slots whose id occurs in
+ * excl[r, 0:e) before that row's first VL_MAXINT become the empty pair.
+ * ids/dists may be strided views (queue.py:47-53 passes the queue tail). */
+int vl_punchout_excluded(int32_t *ids, float *dists, int64_t rows, int64_t cols,
+                         int64_t ids_stride, int64_t dists_stride,
+                         const int32_t *excl, int64_t excl_cols, int64_t excl_stride,
+                         void *stream);
+
+/* index_by_tensor (kernels.py:554-559) for 4-byte elements:
+ * out[r, c] = a[r, index[r, c]], index is int64 as torch.sort returns it. */
+int vl_index_by_tensor(const void *a, const int64_t *index, void *out,
+                       int64_t rows, int64_t cols, void *stream);
+
+/* ---- sorted queues (vectorlink_gpu/queue.py) -------------------------- */
+
+/* index_sort (utils.py:44-53): order each row by (distance asc, id asc). */
+int vl_index_sort(int32_t *ids, float *dists, int64_t rows, int64_t cols, void *stream);
+
+/* punchout_duplicates_ (kernels.py:400-406): dedup_pairs, then order by
+ * distance keeping the previous order on ties.  In place. */
+int vl_punchout_duplicates(int32_t *ids, float *dists, int64_t rows, int64_t cols, void *stream);
+
+/* queue_sort (queue.py:15-18) = index_sort then punchout_duplicates_. */
+int vl_queue_sort(int32_t *ids, float *dists, int64_t rows, int64_t cols, void *stream);
+
+/* Queue.insert (queue.py:37-61): copy m candidates per row into slots
+ * [length, length+m), punch those that occur in the exclusion row (may be
+ * NULL), queue_sort the whole row of `capacity` slots.  When changed is not
+ * NULL it receives, as bytes, indices[:, :length] != the ids before. */
+int vl_queue_insert(int32_t *q_ids, float *q_dists, int64_t rows, int64_t capacity,
+                    int64_t length, const int32_t *cand_ids, const float *cand_dists,
+                    int64_t m, const int32_t *excl, int64_t excl_cols,
+                    uint8_t *changed, void *stream);
+
+/* Queue.pop_n_ids (queue.py:87-95): out[r, 0:take) = ids[r, 0:take); those
+ * slots become the empty pair; nothing is re-sorted. */
+int vl_queue_pop(int32_t *q_ids, float *q_dists, int64_t rows, int64_t capacity,
+                 int64_t take, int32_t *out, void *stream);
+
+/* add_new_to_seen_ (utils.py:61-82): append visit[:, 0:n) at the first
+ * column that is empty in every row, then sort + dedup + sort each row.
+ * host_status receives 1 (updated) or 0 (no free column: the reference
+ * returns None and seen is left as it was).  Synchronises the stream.
+ * workspace: 8 bytes. */
+int vl_seen_add(int32_t *seen, int64_t rows, int64_t cols,
+                const int32_t *visit, int64_t n_visit,
+                void *workspace, int *host_status, void *stream);
+
+/* ---- beam search (ann.py:38-93 closest_vectors) ----------------------- */
+
+typedef struct vl_beam_params {
+    int64_t n_rows;               /* queries in this batch */
+    int64_t dim;
+    int64_t n_vectors;
+    int64_t width;                /* columns of the neighbour table passed in */
+    int64_t queue_capacity;       /* search queue row size */
+    int64_t queue_length;         /* search queue .length */
+    int64_t beam_size;            /* config["beam_size"] */
+    int64_t parallel_visit_count;
+    int64_t visit_queue_factor;
+    int64_t exclude_factor;
+    int64_t speculative_readahead;
+    int64_t excl_cols;            /* columns of the exclusion tensor, 0 if none */
+} vl_beam_params;
+
+int64_t vl_beam_workspace_bytes(const vl_beam_params *p);
+
+/* Runs the whole loop of closest_vectors on the search queue in place and
+ * returns the number of iterations (a multiple of speculative_readahead) or
+ * a negative error.  Synchronises the stream every speculative_readahead
+ * iterations to read the batch-wide "any row changed" flag, as the
+ * reference does (ann.py:90-91).  Rows of the search queue are exact on
+ * [:, :queue_length]; slots beyond are unspecified. */
+int64_t vl_closest_vectors(const vl_beam_params *p,
+                           const float *queries, const float *vectors,
+                           const int32_t *beams,
+                           int32_t *q_ids, float *q_dists,
+                           const int32_t *exclude,
+                           void *workspace, int64_t workspace_bytes,
+                           void *stream);
+
+/* ---- pruning (kernels.py:441-468 prune_) ------------------------------ */
+
+/* For every x and slot j: y = beams[x,j], z = beams[y,0]; if z occurs in row
+ * x at (last) slot i and d[x,i] > d[x,j] and d[x,i] > d[y,0], slot (x,i)
+ * becomes the empty pair; then each row is ordered by distance.  Every
+ * decision reads the tables as passed in (the reference mutates in place
+ * while other blocks read); results go to the *_out tables. */
+int vl_prune(const int32_t *beams, const float *dists, int64_t n, int64_t width,
+             int32_t *beams_out, float *dists_out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VLGPU_H */

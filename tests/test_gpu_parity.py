@@ -1,0 +1,370 @@
+"""GPU parity: every libvlgpu entry point (reached through the vectorlink_gpu
+Python surface, i.e. through the C ABI) against the CPU oracle on the same
+seeded inputs.  ids must match exactly; distances are compared bit for bit
+because the kernels and the oracle share one documented summation order (the
+contract is rtol 1e-5 / atol 1e-6; bit equality is the stronger statement)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+M = orc.MAXINT
+F = orc.MAXFLOAT
+DEV = "cuda"
+
+
+def unit(rng, n, d):
+    v = rng.standard_normal((n, d)).astype(np.float32)
+    return v / np.linalg.norm(v, axis=1, keepdims=True)
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+def bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+def cfg(**kw):
+    c = dict(orc.DEFAULT_CONFIG)
+    c.update(kw)
+    return c
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+# ---------------------------------------------------------------- distances
+@pytest.mark.parametrize("dim", [4, 20, 64, 100, 128, 130, 256, 384, 768, 1024, 1536, 2048, 2052, 3000])
+def test_gather_distances_bit_exact(dim):
+    say(f"gather_distances dim={dim}")
+    from vectorlink_gpu.kernels import calculate_distances, gather_distances
+
+    rng = np.random.default_rng(dim)
+    n, w = 300, 37
+    v = unit(rng, n, dim)
+    beams = rng.integers(0, n, (n, w)).astype(np.int32)
+    beams[rng.random((n, w)) < 0.1] = M
+    want = orc.calculate_distances(v, beams)
+    got = host(calculate_distances(dev(v), dev(beams)))
+    assert np.array_equal(bits(got), bits(want))
+    # against float64, the contract's tolerance
+    safe = np.where(beams == M, 0, beams)
+    ref = np.clip((1 - np.einsum("nd,nwd->nw", v.astype(np.float64), v[safe].astype(np.float64))) / 2, 0, 1)
+    real = beams != M
+    assert np.allclose(got[real], ref[real], rtol=1e-5, atol=1e-6)
+    assert (got[~real] == F).all()
+    # separate query tensor, ids out of range read as empty
+    q = unit(rng, 50, dim)
+    ids = rng.integers(0, n, (50, 9)).astype(np.int32)
+    ids[0, 0] = n + 5
+    ids[1, 1] = -3
+    got2 = host(gather_distances(dev(q), dev(v), dev(ids)))
+    for r in range(50):
+        for c in range(9):
+            if 0 <= ids[r, c] < n:
+                assert got2[r, c] == orc.distance(v[ids[r, c]], q[r])
+            else:
+                assert got2[r, c] == F
+
+
+@pytest.mark.parametrize("dim,w,nv", [(128, 64, 4), (768, 128, 4), (96, 24, 3), (1536, 48, 2), (50, 7, 5)])
+def test_search_from_seeds(dim, w, nv):
+    say(f"search_from_seeds dim={dim} w={w} nv={nv}")
+    from vectorlink_gpu.kernels import search_from_seeds
+
+    rng = np.random.default_rng(dim + w)
+    n, b = 500, 70
+    v = unit(rng, n, dim)
+    q = unit(rng, b, dim)
+    beams = rng.integers(0, n, (n, w)).astype(np.int32)
+    beams[rng.random((n, w)) < 0.05] = M
+    visit = rng.integers(0, n, (b, nv)).astype(np.int32)
+    visit[rng.random((b, nv)) < 0.2] = M
+    wi, wd = orc.search_from_seeds(q, visit, beams, v)
+    gi, gd = search_from_seeds(dev(q), dev(visit), dev(beams), dev(v))
+    assert np.array_equal(host(gi), wi)
+    assert np.array_equal(bits(host(gd)), bits(wd))
+
+
+def test_circulants():
+    from vectorlink_gpu.utils import generate_circulant_beams, generate_queue_circulants, primes
+
+    assert np.array_equal(host(primes(965)), orc.all_primes())
+    for n, k in [(10, 4), (7, 4), (4096, 64), (1000, 72), (977, 700), (5000, 965)]:
+        say(f"circulants n={n} k={k}")
+        got = host(generate_circulant_beams(n, primes(k)))
+        assert np.array_equal(got, orc.generate_circulant_beams(n, orc.primes(k)))
+        got = host(generate_queue_circulants(33, n, primes(k)))
+        assert np.array_equal(got, orc.generate_queue_circulants(33, n, orc.primes(k)))
+
+
+# ---------------------------------------------------------------- id-list kernels
+def random_rows(rng, rows, cols, n_ids, n_dist, p_sent=0.15):
+    ids = rng.integers(0, n_ids, (rows, cols)).astype(np.int32)
+    d = (rng.integers(0, n_dist, (rows, cols)) / np.float32(n_dist)).astype(np.float32)
+    s = rng.random((rows, cols)) < p_sent
+    ids[s] = M
+    d[s] = F
+    return ids, d
+
+
+@pytest.mark.parametrize("cols", [1, 2, 3, 8, 63, 64, 65, 320, 352, 640, 704, 1000, 1024, 2500, 4096])
+def test_sorts_and_dedup(cols):
+    say(f"sort/dedup cols={cols}")
+    from vectorlink_gpu import kernels as K
+    from vectorlink_gpu.utils import index_sort, queue_sort
+
+    rng = np.random.default_rng(cols)
+    rows = 40
+    ids, d = random_rows(rng, rows, cols, max(3, cols // 3), 7)
+    wi, wd = orc.index_sort(ids, d)
+    gi, gd = index_sort(dev(ids), dev(d))
+    assert np.array_equal(host(gi), wi) and np.array_equal(bits(host(gd)), bits(wd))
+
+    wi, wd = orc.queue_sort(ids, d)
+    gi, gd = queue_sort(dev(ids), dev(d))
+    assert np.array_equal(host(gi), wi) and np.array_equal(bits(host(gd)), bits(wd))
+
+    # punchout_duplicates_ on rows ordered by id (neighbouring duplicates)
+    sid = np.sort(ids, axis=1)
+    wi, wd = orc.punchout_duplicates_(sid, d)
+    ti, td = dev(sid), dev(d)
+    K.punchout_duplicates_(ti, td)
+    assert np.array_equal(host(ti), wi) and np.array_equal(bits(host(td)), bits(wd))
+
+    a, b = sid.copy(), d.copy()
+    orc.dedup_tensor_pair_(a, b)
+    ti, td = dev(sid), dev(d)
+    K.dedup_tensor_pair_(ti, td)
+    assert np.array_equal(host(ti), a) and np.array_equal(bits(host(td)), bits(b))
+    c = sid.copy()
+    orc.dedup_tensor_(c)
+    ti = dev(sid)
+    K.dedup_tensor_(ti)
+    assert np.array_equal(host(ti), c)
+
+
+def test_queue_sort_odd_distances():
+    # distances outside [0,1]: negative, beyond MAXFLOAT, infinities; -0.0 comes back as +0.0
+    from vectorlink_gpu.utils import queue_sort
+
+    ids = np.array([[4, 9, 2, 7, M, 5, 5, 3, 8]], np.int32)
+    d = np.array([[-1.5, np.inf, 3.0e38, 0.0, F, 1e-30, 1e-30, -0.0, F]], np.float32)
+    wi, wd = orc.queue_sort(ids, d)
+    gi, gd = queue_sort(dev(ids), dev(d))
+    assert np.array_equal(host(gi), wi)
+    assert np.array_equal(host(gd), wd)  # value equality: -0.0 == +0.0
+
+
+def test_punchout_excluded_strided_view():
+    from vectorlink_gpu.kernels import punchout_excluded_
+
+    rng = np.random.default_rng(5)
+    rows, cap, length, m, e = 30, 50, 12, 30, 9
+    ids, d = random_rows(rng, rows, cap, 25, 5)
+    excl = rng.integers(0, 25, (rows, e)).astype(np.int32)
+    excl[rng.random((rows, e)) < 0.2] = M
+    wi, wd = ids.copy(), d.copy()
+    ti, td = np.ascontiguousarray(wi[:, length:length + m]), np.ascontiguousarray(wd[:, length:length + m])
+    orc.punchout_excluded_(ti, td, excl)
+    wi[:, length:length + m], wd[:, length:length + m] = ti, td
+    gi, gd = dev(ids), dev(d)
+    punchout_excluded_(gi.narrow(1, length, m), gd.narrow(1, length, m), dev(excl))
+    assert np.array_equal(host(gi), wi) and np.array_equal(bits(host(gd)), bits(wd))
+    assert (wi != ids).any()
+
+
+def test_index_by_tensor():
+    from vectorlink_gpu.kernels import index_by_tensor
+
+    rng = np.random.default_rng(6)
+    a = rng.integers(0, 1000, (19, 77)).astype(np.int32)
+    b = np.stack([rng.permutation(77) for _ in range(19)])
+    assert np.array_equal(host(index_by_tensor(dev(a), dev(b))), np.take_along_axis(a, b, axis=1))
+    f = rng.random((19, 77)).astype(np.float32)
+    assert np.array_equal(host(index_by_tensor(dev(f), dev(b))), np.take_along_axis(f, b, axis=1))
+
+
+# ---------------------------------------------------------------- Queue
+def test_queue_kat():
+    from vectorlink_gpu import Queue
+
+    q = Queue(1, 4, 8)
+    q.insert(dev(np.array([[5, 3, 5, 9]], np.int32)), dev(np.array([[.3, .1, .3, .2]], np.float32)))
+    assert host(q.indices).tolist() == [[3, 9, 5, M, M, M, M, M]]
+    mask = q.insert(dev(np.array([[7, 3, 2, M]], np.int32)), dev(np.array([[.05, .1, .2, F]], np.float32)),
+                    exclude=dev(np.array([[2, M]], np.int32)), output_update=True)
+    assert host(q.indices).tolist() == [[7, 3, 9, 5, M, M, M, M]]
+    assert host(q.distances)[0, :4].tolist() == [np.float32(x) for x in (.05, .1, .2, .3)]
+    assert host(mask).tolist() == [[True, True, True, True]]
+    assert host(q.pop_n_ids(2)).tolist() == [[7, 3]]
+    assert host(q.indices).tolist() == [[M, M, 9, 5, M, M, M, M]]
+    assert host(q.distances)[0, 0] == F
+
+
+@pytest.mark.parametrize("length,m,cap,e", [(4, 6, 10, 0), (64, 256, 320, 1), (96, 256, 352, 480), (128, 512, 640, 1),
+                                           (192, 512, 704, 960), (20, 30, 64, 7), (64, 128, 320, 3)])
+def test_queue_insert_pop_sequence(length, m, cap, e):
+    say(f"queue sequence length={length} m={m} cap={cap} excl={e}")
+    from vectorlink_gpu import Queue
+
+    rng = np.random.default_rng(length * 7 + m)
+    rows = 25
+    table = rng.random(400).astype(np.float32)  # an id always carries the same distance
+    table[100:140] = table[100]
+    oq = orc.Queue(rows, length, cap)
+    gq = Queue(rows, length, cap)
+    for step in range(6):
+        ids = rng.integers(0, 400, (rows, m)).astype(np.int32)
+        d = table[ids]
+        s = rng.random((rows, m)) < 0.1
+        ids[s], d[s] = M, F
+        ex = None
+        if e:
+            ex = rng.integers(0, 400, (rows, e)).astype(np.int32)
+            ex.sort(axis=1)
+            ex[:, e // 2 + 1:] = M
+        upd = step % 2 == 1
+        wm = oq.insert(ids, d, exclude=ex, output_update=upd)
+        gm = gq.insert(dev(ids), dev(d), exclude=None if ex is None else dev(ex), output_update=upd)
+        assert np.array_equal(host(gq.indices), oq.indices), step
+        assert np.array_equal(bits(host(gq.distances)), bits(oq.distances))
+        if upd:
+            assert np.array_equal(host(gm), wm)
+        if step == 3:
+            assert np.array_equal(host(gq.pop_n_ids(3)), oq.pop_n_ids(3))
+            assert np.array_equal(host(gq.indices), oq.indices)
+
+
+def test_seen_add_sequence():
+    from vectorlink_gpu.utils import add_new_to_seen_
+
+    rng = np.random.default_rng(8)
+    rows, cols, nv = 20, 22, 4
+    so = np.full((rows, cols), M, np.int32)
+    sg = dev(so)
+    alive_o, alive_g = so, sg
+    for step in range(30):
+        visit = rng.integers(0, 600, (rows, nv)).astype(np.int32)
+        visit[rng.random((rows, nv)) < 0.2] = M
+        alive_o = orc.add_new_to_seen_(so, visit)
+        alive_g = add_new_to_seen_(sg, dev(visit))
+        assert (alive_o is None) == (alive_g is None), step
+        assert np.array_equal(host(sg), so), step
+        if alive_o is None:
+            break
+    assert alive_o is None  # the list did fill up
+
+
+# ---------------------------------------------------------------- prune
+def test_prune():
+    from vectorlink_gpu.kernels import prune_
+
+    b = np.array([[1, 2], [2, 0], [1, 0]], np.int32)
+    d = np.array([[.1, .3], [.05, .1], [.05, .3]], np.float32)
+    gb, gd = prune_(dev(b), dev(d))
+    assert host(gb).tolist() == [[1, M], [2, 0], [1, 0]]
+    assert host(gd)[0].tolist() == [np.float32(.1), F]
+    rng = np.random.default_rng(9)
+    for n, w, dim in [(200, 6, 8), (3000, 64, 16), (1500, 128, 8), (500, 24, 12)]:
+        say(f"prune n={n} w={w}")
+        v = unit(rng, n, dim)
+        beams = np.stack([rng.choice(n, w, replace=False) for _ in range(n)]).astype(np.int32)
+        beams[rng.random((n, w)) < 0.03] = M
+        dd = orc.calculate_distances(v, beams)
+        beams, dd = orc.queue_sort(beams, dd)
+        wb, wd = orc.prune_(beams, dd)
+        gb, gd = prune_(dev(beams), dev(dd))
+        assert np.array_equal(host(gb), wb) and np.array_equal(bits(host(gd)), bits(wd))
+        assert (wb != beams).any()
+
+
+# ---------------------------------------------------------------- beam search
+BEAM_CASES = [
+    # n, dim, beam, bqf, pv, vqf, ef, ra
+    (64, 8, 4, 2, 2, 3, 5, 5),
+    (600, 32, 8, 2, 4, 3, 5, 5),
+    (500, 128, 32, 2, 4, 3, 5, 5),
+    (300, 12, 5, 2, 3, 2, 1, 2),   # small visited list: fills up, the visit queue stops being fed
+    (200, 10, 2, 2, 4, 1, 2, 3),   # visit queue shorter than the visit count
+    (400, 768, 16, 2, 4, 3, 5, 5),
+]
+
+
+@pytest.mark.parametrize("n,dim,beam,bqf,pv,vqf,ef,ra", BEAM_CASES)
+@pytest.mark.parametrize("fused", [True, False])
+def test_closest_vectors_build_step(n, dim, beam, bqf, pv, vqf, ef, ra, fused):
+    say(f"closest_vectors n={n} dim={dim} beam={beam} fused={fused}")
+    from vectorlink_gpu import Queue
+    from vectorlink_gpu.ann import closest_vectors, closest_vectors_stepwise, excluding_self
+
+    rng = np.random.default_rng(n + dim)
+    v = unit(rng, n, dim)
+    c = cfg(beam_size=beam, beam_queue_factor=bqf, parallel_visit_count=pv, visit_queue_factor=vqf,
+            exclude_factor=ef, speculative_readahead=ra)
+    ql = beam * bqf
+    beams = orc.generate_circulant_beams(n, orc.primes(ql))
+    d = orc.calculate_distances(v, beams)
+    lo, hi = 3, n - 2
+    oq = orc.Queue(hi - lo, ql, ql + ql * pv)
+    oq.insert(beams[lo:hi], d[lo:hi])
+    t_want = orc.closest_vectors(v[lo:hi], oq, v, beams, c, orc.excluding_self(lo, hi))
+
+    gv, gb = dev(v), dev(beams)
+    gq = Queue(hi - lo, ql, ql + ql * pv)
+    gq.insert(gb[lo:hi], dev(d)[lo:hi])
+    fn = closest_vectors if fused else closest_vectors_stepwise
+    t_got = fn(gv[lo:hi], gq, gv, gb, c, excluding_self(lo, hi))
+    assert t_got == t_want
+    assert np.array_equal(host(gq.indices)[:, :ql], oq.indices[:, :ql])
+    assert np.array_equal(bits(host(gq.distances)[:, :ql]), bits(oq.distances[:, :ql]))
+
+
+def test_generate_ann_and_search_against_oracle():
+    say("generate_ann + search, n=1500")
+    from vectorlink_gpu import ANN
+
+    rng = np.random.default_rng(14)
+    n, dim = 1500, 24
+    v = unit(rng, n, dim)
+    kw = dict(beam_size=12, beam_queue_factor=2, recall_search_queue_factor=2, batch_size=400, optimization_loops=2)
+    c = cfg(**kw)
+    wb, wd = orc.generate_ann(v, c)
+    ann = ANN(dev(v), **kw)
+    assert np.array_equal(host(ann.beams), wb)
+    assert np.array_equal(bits(host(ann.distances)), bits(wd))
+    qv = unit(rng, 100, dim)
+    res = ann.search(dev(qv))
+    want = orc.search(v, wb, qv, c)
+    L = want.length
+    assert np.array_equal(host(res.indices)[:, :L], want.indices[:, :L])
+    assert np.array_equal(bits(host(res.distances)[:, :L]), bits(want.distances[:, :L]))
+    assert ann.recall(300) == orc.ann_calculate_recall(v, wb, c, sample=v[:300])
+    # a longer search queue than configured
+    res = ann.search(dev(qv), queue_size=40)
+    want = orc.search(v, wb, qv, c, queue_size=40)
+    assert np.array_equal(host(res.indices)[:, :40], want.indices[:, :40])
+    # resume from a stored graph (ann.py:391-396)
+    again = ANN(dev(v), beams=ann.beams, **kw)
+    assert np.array_equal(bits(host(again.distances)), bits(wd))
+
+
+def test_generate_ann_stale_distance_mode():
+    from vectorlink_gpu.ann import generate_ann
+
+    rng = np.random.default_rng(15)
+    v = unit(rng, 400, 12)
+    c = cfg(beam_size=6, beam_queue_factor=2, batch_size=150, optimization_loops=2, prune=True)
+    wb, wd = orc.generate_ann(v, c, stale_distances=True)
+    gb, gd = generate_ann(dev(v), c, stale_distances=True)
+    assert np.array_equal(host(gb), wb) and np.array_equal(bits(host(gd)), bits(wd))

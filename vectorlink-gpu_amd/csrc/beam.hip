@@ -1,0 +1,351 @@
+// The beam-search loop of closest_vectors (vectorlink_gpu/ann.py:38-93) for
+// gfx950.
+//
+// The reference runs ~50 torch ops / Numba launches and at least two blocking
+// host round trips per iteration.  Here an iteration is two launches:
+//   expand  (dist.hip)  pop the visit-queue heads, gather their neighbour
+//                       lists, evaluate the candidate distances;
+//   merge   (this file) one workgroup per query row: insert the candidates
+//                       into the search queue (Queue.insert, queue.py:37-61),
+//                       record the visited ids (add_new_to_seen_,
+//                       utils.py:61-82) and refill the visit queue with the
+//                       candidates not yet visited.
+// Batch-wide state (first free visited-list column, "any row changed") lives
+// in a device control block; the host only reads the changed flag every
+// speculative_readahead iterations, the cadence at which the reference tests
+// for progress (ann.py:68,90-91).
+#include "beam_ctrl.h"
+#include "rowsort.h"
+
+int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors, int64_t n_vectors,
+                     int64_t dim, const int32_t *ids, const int32_t *visit, int64_t n_visit,
+                     const int32_t *beams, int64_t n_nodes, int64_t width, int64_t m,
+                     int32_t *idx_out, float *dist_out, BeamCtrl *ctrl, int iter, int readahead,
+                     int seen_cols, int64_t visit_stride, hipStream_t st);
+
+namespace {
+
+constexpr int kMaxVisit = 64;  // parallel_visit_count handled by one wavefront
+
+struct MergeArgs {
+    BeamCtrl *ctrl;
+    int iter;
+    int readahead;
+    int64_t n_rows;
+    const int32_t *cand_ids;
+    const float *cand_d;
+    int m;
+    int32_t *q_ids;
+    float *q_d;
+    int cap, L, Ps;
+    const int32_t *excl;
+    int excl_cols;
+    int32_t *v_ids;
+    float *v_d;
+    int VL, Vt, Pv;
+    int32_t *seen;
+    int32_t *seen_count;
+    int E;
+};
+
+__device__ inline bool sorted_contains(const int32_t *a, int n, int32_t v) {
+    int lo = 0, hi = n;
+    while (lo < hi) {
+        int mid = (lo + hi) >> 1;
+        if (a[mid] < v) lo = mid + 1;
+        else hi = mid;
+    }
+    return lo < n && a[lo] == v;
+}
+__device__ inline int lower_bound(const int32_t *a, int n, int32_t v) {
+    int lo = 0, hi = n;
+    while (lo < hi) {
+        int mid = (lo + hi) >> 1;
+        if (a[mid] < v) lo = mid + 1;
+        else hi = mid;
+    }
+    return lo;
+}
+
+__global__ __launch_bounds__(kQueueThreads) void beam_init_kernel(BeamCtrl *ctrl, int64_t n_rows, const int32_t *q_ids,
+                                                                 const float *q_d, int cap, int head, int32_t *v_ids,
+                                                                 float *v_d, int VL, int32_t *seen_count) {
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t == 0) {
+        ctrl->stop = 0;
+        ctrl->reserved = 0;
+        ctrl->first[0] = ctrl->first[1] = 0;
+    }
+    if (t < 64) ctrl->changed[t] = 0;
+    if (t < n_rows) seen_count[t] = 0;
+    if (t < n_rows * VL) {  // Queue.initialize_from_queue, queue.py:30-35
+        int64_t r = t / VL;
+        int i = (int)(t % VL);
+        v_ids[t] = i < head ? q_ids[r * cap + i] : VL_MAXINT;
+        v_d[t] = i < head ? q_d[r * cap + i] : VL_MAXFLOAT;
+    }
+}
+
+__global__ __launch_bounds__(kQueueThreads) void beam_merge_kernel(MergeArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int Pmax = a.Ps > a.Pv ? a.Ps : a.Pv;
+    uint64_t *keys = reinterpret_cast<uint64_t *>(smem);
+    int32_t *before = reinterpret_cast<int32_t *>(keys + Pmax);
+    int32_t *seen_a = before + a.L;
+    int32_t *seen_b = seen_a + a.E;
+    int32_t *exl = seen_b + a.E;
+    __shared__ PlaceScratch ps;
+    __shared__ int n_ex_s;
+    __shared__ int32_t newv[kMaxVisit];
+    __shared__ int n_new_s;
+
+    BeamCtrl *c = a.ctrl;
+    if (c->stop) return;
+    const int t = a.iter;
+    const int64_t row = blockIdx.x;
+    int cnt = a.seen_count[row];
+    int *first_next = &c->first[(t + 1) & 1];
+    if (t >= 2 && c->first[(t - 1) & 1] >= a.E) {
+        // the visit queue is no longer fed: every candidate of this iteration is
+        // empty and no queue changes; keep the running maximum current
+        if (threadIdx.x == 0) atomicMax(first_next, cnt);
+        return;
+    }
+    const int first = c->first[t & 1];
+    const bool seen_full = first >= a.E;  // add_new_to_seen_ returns None now (utils.py:68-69)
+    const bool checking = (t % a.readahead) == 0;
+
+    // ---- search_queue.insert(candidates, exclude) : ann.py:75-80 -----------
+    if (threadIdx.x == 0) n_ex_s = a.excl ? a.excl_cols : 0;
+    __syncthreads();
+    if (a.excl) {
+        const int32_t *ex = a.excl + row * a.excl_cols;
+        for (int i = threadIdx.x; i < a.excl_cols; i += blockDim.x) {
+            int32_t e = ex[i];
+            exl[i] = e;
+            if (e == VL_MAXINT) atomicMin(&n_ex_s, i);
+        }
+    }
+    int32_t *qi = a.q_ids + row * a.cap;
+    float *qd = a.q_d + row * a.cap;
+    const int32_t *ci = a.cand_ids + row * a.m;
+    const float *cd = a.cand_d + row * a.m;
+    for (int i = threadIdx.x; i < a.L; i += blockDim.x) before[i] = qi[i];
+    __syncthreads();
+    const int n_ex = n_ex_s;
+    for (int i = threadIdx.x; i < a.Ps; i += blockDim.x) {
+        uint64_t k = kPadKey;
+        if (i < a.cap) {
+            int32_t id;
+            float d;
+            if (i >= a.L && i < a.L + a.m) {
+                id = ci[i - a.L];
+                d = cd[i - a.L];
+                bool hit = false;
+                for (int e = 0; e < n_ex; ++e) hit |= (exl[e] == id);
+                if (hit) {
+                    id = VL_MAXINT;
+                    d = VL_MAXFLOAT;
+                }
+            } else {
+                id = qi[i];
+                d = qd[i];
+            }
+            k = vl_make_key(id, d);
+        }
+        keys[i] = k;
+    }
+    block_bitonic_sort(keys, a.Ps);
+    block_place3(keys, a.cap, a.cap, qi, qd, &ps, before, a.L, nullptr,
+                 checking ? &c->changed[(t / a.readahead) & 63] : nullptr);
+
+    if (seen_full) {
+        if (threadIdx.x == 0) atomicMax(first_next, cnt);
+        return;
+    }
+
+    // ---- add_new_to_seen_(seen, visited) : utils.py:61-82 -------------------
+    // The row is kept sorted, duplicate free and packed at the front, which is
+    // what sort + dedup + sort leaves; `cnt` ids are in use.
+    int32_t *srow = a.seen + row * a.E;
+    const int32_t *vrow_i = a.v_ids + row * a.VL;
+    const float *vrow_d = a.v_d + row * a.VL;
+    for (int i = threadIdx.x; i < cnt; i += blockDim.x) seen_a[i] = srow[i];
+    if (threadIdx.x == 0) n_new_s = 0;
+    __syncthreads();
+    const int n_add = min(a.E - first, a.Vt);  // utils.py:73-75
+    if (threadIdx.x < kWave) {
+        const int j = threadIdx.x;
+        int32_t x = j < n_add ? vrow_i[j] : VL_MAXINT;
+        bool valid = j < n_add && x != VL_MAXINT && !sorted_contains(seen_a, cnt, x);
+        for (int i = 0; i < j && valid; ++i)
+            if (vrow_i[i] == x) valid = false;
+        uint64_t vm = __ballot(valid);
+        // ascending rank among the valid new ids
+        int rank = 0;
+        for (int i = 0; i < n_add; ++i) {
+            int32_t y = vrow_i[i];
+            if (((vm >> i) & 1) && y < x) ++rank;
+        }
+        if (valid) newv[rank] = x;
+        if (j == 0) n_new_s = __popcll(vm);
+    }
+    __syncthreads();
+    const int n_new = n_new_s;
+    for (int p = threadIdx.x; p < cnt; p += blockDim.x) {
+        int32_t v = seen_a[p];
+        int shift = 0;
+        for (int i = 0; i < n_new; ++i) shift += newv[i] < v;
+        seen_b[p + shift] = v;
+    }
+    if (threadIdx.x < n_new) seen_b[lower_bound(seen_a, cnt, newv[threadIdx.x]) + threadIdx.x] = newv[threadIdx.x];
+    __syncthreads();
+    cnt += n_new;
+    for (int i = threadIdx.x; i < cnt; i += blockDim.x) srow[i] = seen_b[i];
+    if (threadIdx.x == 0) {
+        a.seen_count[row] = cnt;
+        atomicMax(first_next, cnt);
+    }
+
+    // ---- visit_queue.insert(candidates, exclude=seen) : ann.py:85-88 --------
+    // slots [0, Vt) were popped at the start of this iteration (queue.py:87-95)
+    for (int i = threadIdx.x; i < a.Pv; i += blockDim.x) {
+        uint64_t k = kPadKey;
+        if (i < a.VL + a.m) {
+            int32_t id = VL_MAXINT;
+            float d = VL_MAXFLOAT;
+            if (i >= a.VL) {
+                id = ci[i - a.VL];
+                d = cd[i - a.VL];
+                if (sorted_contains(seen_b, cnt, id)) {
+                    id = VL_MAXINT;
+                    d = VL_MAXFLOAT;
+                }
+            } else if (i >= a.Vt) {
+                id = vrow_i[i];
+                d = vrow_d[i];
+            }
+            k = vl_make_key(id, d);
+        }
+        keys[i] = k;
+    }
+    block_bitonic_sort(keys, a.Pv);
+    block_place3(keys, a.VL + a.m, a.VL, a.v_ids + row * a.VL, a.v_d + row * a.VL, &ps, nullptr, 0, nullptr,
+                 nullptr);
+}
+
+struct BeamLayout {
+    int64_t m, VL, Vt, E, head;
+    int64_t off_cand_ids, off_cand_d, off_v_ids, off_v_d, off_seen, off_seen_count, off_ctrl, total;
+};
+
+inline int64_t align256(int64_t x) { return (x + 255) & ~255ll; }
+
+int beam_layout(const vl_beam_params *p, BeamLayout *l) {
+    VL_REQUIRE(p, "null params");
+    VL_REQUIRE(p->n_rows >= 0 && p->dim > 0 && p->n_vectors > 0 && p->width > 0, "bad sizes");
+    VL_REQUIRE(p->beam_size > 0 && p->parallel_visit_count > 0 && p->visit_queue_factor > 0 &&
+                   p->exclude_factor > 0 && p->speculative_readahead > 0,
+               "configuration values must be positive");
+    VL_REQUIRE(p->queue_length > 0 && p->queue_length < p->queue_capacity, "queue length must be below its capacity");
+    VL_REQUIRE(p->n_vectors < (1ll << 30), "ids must stay below 2^30");
+    l->VL = p->visit_queue_factor * p->beam_size;                                      // ann.py:51
+    l->Vt = l->VL < p->parallel_visit_count ? l->VL : p->parallel_visit_count;         // queue.py:89
+    l->m = l->Vt * p->width;
+    l->E = p->exclude_factor * l->VL;                                                  // ann.py:55
+    l->head = p->queue_length < l->VL ? p->queue_length : l->VL;                       // queue.py:31
+    VL_REQUIRE(l->Vt <= kMaxVisit, "parallel_visit_count above %d is not supported", kMaxVisit);
+    VL_REQUIRE(p->queue_length + l->m <= p->queue_capacity,
+               "search queue capacity %lld cannot take %lld candidates after its %lld slots",
+               (long long)p->queue_capacity, (long long)l->m, (long long)p->queue_length);
+    VL_REQUIRE(p->queue_capacity <= kMaxRowSlots && l->VL + l->m <= kMaxRowSlots && l->E <= kMaxRowSlots,
+               "queue rows above %d slots are not supported", kMaxRowSlots);
+    VL_REQUIRE(p->excl_cols >= 0 && p->excl_cols <= 1024, "exclusion rows above 1024 ids are not supported here");
+    int64_t o = 0;
+    l->off_cand_ids = o; o = align256(o + p->n_rows * l->m * 4);
+    l->off_cand_d = o; o = align256(o + p->n_rows * l->m * 4);
+    l->off_v_ids = o; o = align256(o + p->n_rows * l->VL * 4);
+    l->off_v_d = o; o = align256(o + p->n_rows * l->VL * 4);
+    l->off_seen = o; o = align256(o + p->n_rows * l->E * 4);
+    l->off_seen_count = o; o = align256(o + p->n_rows * 4);
+    l->off_ctrl = o; o = align256(o + (int64_t)sizeof(BeamCtrl));
+    l->total = o;
+    return VL_OK;
+}
+
+}  // namespace
+
+VL_EXPORT int64_t vl_beam_workspace_bytes(const vl_beam_params *p) {
+    BeamLayout l;
+    int rc = beam_layout(p, &l);
+    return rc < 0 ? rc : l.total;
+}
+
+VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queries, const float *vectors,
+                                     const int32_t *beams, int32_t *q_ids, float *q_dists,
+                                     const int32_t *exclude, void *workspace, int64_t workspace_bytes,
+                                     void *stream) {
+    BeamLayout l;
+    int rc = beam_layout(p, &l);
+    if (rc < 0) return rc;
+    if (p->n_rows == 0) return 0;
+    VL_REQUIRE(queries && vectors && beams && q_ids && q_dists && workspace, "null pointer");
+    VL_REQUIRE(((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
+    if (workspace_bytes < l.total) {
+        vl_set_error("workspace of %lld bytes is smaller than the %lld needed", (long long)workspace_bytes,
+                     (long long)l.total);
+        return VL_ERR_WORKSPACE;
+    }
+    VL_REQUIRE(p->n_rows * (l.VL > l.m ? l.VL : l.m) < (1ll << 40), "batch too large");
+    hipStream_t st = (hipStream_t)stream;
+    char *ws = (char *)workspace;
+    int32_t *cand_ids = (int32_t *)(ws + l.off_cand_ids);
+    float *cand_d = (float *)(ws + l.off_cand_d);
+    int32_t *v_ids = (int32_t *)(ws + l.off_v_ids);
+    float *v_d = (float *)(ws + l.off_v_d);
+    int32_t *seen = (int32_t *)(ws + l.off_seen);
+    int32_t *seen_count = (int32_t *)(ws + l.off_seen_count);
+    BeamCtrl *ctrl = (BeamCtrl *)(ws + l.off_ctrl);
+
+    {
+        int64_t n = p->n_rows * l.VL;
+        if (n < 64) n = 64;
+        if (n < p->n_rows) n = p->n_rows;
+        hipLaunchKernelGGL(beam_init_kernel, dim3((unsigned)((n + kQueueThreads - 1) / kQueueThreads)),
+                           dim3(kQueueThreads), 0, st, ctrl, p->n_rows, q_ids, q_dists, (int)p->queue_capacity,
+                           (int)l.head, v_ids, v_d, (int)l.VL, seen_count);
+        VL_LAUNCH_CHECK("beam_init_kernel");
+    }
+
+    MergeArgs a;
+    a.ctrl = ctrl; a.readahead = (int)p->speculative_readahead; a.n_rows = p->n_rows;
+    a.cand_ids = cand_ids; a.cand_d = cand_d; a.m = (int)l.m;
+    a.q_ids = q_ids; a.q_d = q_dists; a.cap = (int)p->queue_capacity; a.L = (int)p->queue_length;
+    a.Ps = vl_next_pow2(a.cap);
+    a.excl = p->excl_cols > 0 ? exclude : nullptr; a.excl_cols = a.excl ? (int)p->excl_cols : 0;
+    a.v_ids = v_ids; a.v_d = v_d; a.VL = (int)l.VL; a.Vt = (int)l.Vt; a.Pv = vl_next_pow2(l.VL + l.m);
+    a.seen = seen; a.seen_count = seen_count; a.E = (int)l.E;
+    const int Pmax = a.Ps > a.Pv ? a.Ps : a.Pv;
+    const size_t smem = (size_t)Pmax * 8 + (size_t)a.L * 4 + (size_t)a.E * 8 + (size_t)a.excl_cols * 4;
+    VL_REQUIRE(smem <= 60 * 1024, "queues of this size need %zu bytes of LDS (limit 61440)", smem);
+
+    const int R = (int)p->speculative_readahead;
+    int64_t t = 0;
+    for (;;) {
+        for (int r = 0; r < R; ++r) {
+            ++t;
+            rc = vl_launch_expand(queries, p->n_rows, vectors, p->n_vectors, p->dim, nullptr, v_ids, l.Vt, beams,
+                                  p->n_vectors, p->width, l.m, cand_ids, cand_d, ctrl, (int)t, R, (int)l.E, l.VL, st);
+            if (rc < 0) return rc;
+            a.iter = (int)t;
+            hipLaunchKernelGGL(beam_merge_kernel, dim3((unsigned)p->n_rows), dim3(kQueueThreads), smem, st, a);
+            VL_LAUNCH_CHECK("beam_merge_kernel");
+        }
+        int changed = 0;
+        VL_HIP(hipMemcpyAsync(&changed, &ctrl->changed[(t / R) & 63], sizeof(int), hipMemcpyDeviceToHost, st));
+        VL_HIP(hipStreamSynchronize(st));
+        if (!changed) break;  // ann.py:90-91
+        VL_REQUIRE(t < (1ll << 30), "beam search did not terminate");
+    }
+    return t;
+}

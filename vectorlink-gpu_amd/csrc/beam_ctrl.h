@@ -1,0 +1,37 @@
+// Device-side control block of one closest_vectors loop (ann.py:38-93).
+// Batch-wide facts that the reference obtains with host round trips live here
+// so that the per-iteration kernels can be enqueued back to back:
+//   stop        - set once a checking iteration saw no row change (ann.py:90-91)
+//   first[2]    - largest visited-list fill over all rows, double buffered by
+//                 iteration parity; it is the first column that is empty in
+//                 every row (utils.py:63-66) because rows are kept sorted
+//   changed[64] - ring of "some row changed" flags, one per checking iteration
+#pragma once
+#include "vl_common.h"
+
+struct BeamCtrl {
+    int stop;
+    int reserved;
+    int first[2];
+    int changed[64];
+};
+
+// State of iteration t as seen by a kernel launched for it:
+//   2  the loop has ended, do nothing
+//   1  the visited list filled up earlier (add_new_to_seen_ returned None,
+//      utils.py:68-69): the visit queue is no longer fed and pops yield empty ids
+//   0  normal
+// `writer` is true for exactly one thread of the launch, which records stop
+// and clears the ring slot of the next checking iteration.
+__device__ inline int beam_gate(BeamCtrl *c, int t, int R, int E, bool writer) {
+    int stop = c->stop;
+    const bool after_check = t > 1 && ((t - 1) % R) == 0;
+    if (!stop && after_check && c->changed[((t - 1) / R) & 63] == 0) stop = 1;
+    if (stop) {
+        if (writer) c->stop = 1;
+        return 2;
+    }
+    if (writer && ((t - 1) % R) == 0) c->changed[((t - 1) / R + 1) & 63] = 0;
+    if (t >= 2 && c->first[(t - 1) & 1] >= E) return 1;
+    return 0;
+}

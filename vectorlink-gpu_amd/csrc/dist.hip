@@ -1,0 +1,286 @@
+// Gathered cosine distances for gfx950: the replacement of the reference's
+// cuda_distances_kernel (vectorlink_gpu/kernels.py:130-171) and
+// cuda_search_from_seeds_kernel (kernels.py:204-257).
+//
+// The reference launches one thread block per scalar distance.  Here one
+// wavefront owns up to 64 candidate ids (one per lane), keeps the query row in
+// registers, and streams the candidate rows with 16-byte loads, several rows in
+// flight at a time; sentinel candidates are compacted away with a ballot before
+// any row is fetched.  HBM traffic is the candidate rows: 4*dim bytes each.
+//
+// Summation order of one dot product (fixed so that every entry point and the
+// CPU oracle produce the same bits): the row is cut into chunks of 4 floats,
+// chunk c belongs to partial sum c mod 64, a partial sum takes its elements in
+// index order with one fused multiply-add each, and the 64 partial sums are
+// folded pairwise at lane distances 32, 16, 8, 4, 2, 1.  Rows of at most
+// 4*LPR floats (LPR = 16 or 32) are handled by groups of LPR lanes, several
+// rows per wavefront; the missing upper partial sums are zeros, so the result
+// is the same.
+#include "vl_common.h"
+#include "beam_ctrl.h"
+
+namespace {
+
+__device__ __forceinline__ float clamp_distance(float cos_theta) {
+    float r = (1.0f - cos_theta) * 0.5f;  // kernels.py:109
+    if (r < 0.0f) r = 0.0f;               // kernels.py:110-113
+    else if (r > 1.0f) r = 1.0f;
+    return r;
+}
+
+// One wavefront: lane j holds candidate id `my_id` (valid when `ok`); the
+// distance of candidate lane j to the query goes to out_d[j].
+template <int CPL, int LPR, int U>
+__device__ __forceinline__ void wave_distances(const float *__restrict__ q_row,
+                                               const float *__restrict__ vectors, int dim,
+                                               int nchunks, int32_t my_id, bool ok,
+                                               float *__restrict__ out_d) {
+    constexpr int G = kWave / LPR;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int grp = lane / LPR;
+    const int lig = lane % LPR;
+
+    float4 q[CPL];
+    bool cvalid[CPL];
+#pragma unroll
+    for (int i = 0; i < CPL; ++i) {
+        int c = lig + LPR * i;
+        cvalid[i] = c < nchunks;
+        q[i] = cvalid[i] ? reinterpret_cast<const float4 *>(q_row)[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+
+    uint64_t mask = __ballot(ok);
+    while (mask) {
+        int src[U][G];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                if (mask) {
+                    src[u][g] = __builtin_ctzll(mask);
+                    mask &= mask - 1;
+                } else {
+                    src[u][g] = -1;
+                }
+            }
+
+        float4 r[U][CPL];
+        int mysrc[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int s = src[u][0];
+#pragma unroll
+            for (int g = 1; g < G; ++g) s = (grp == g) ? src[u][g] : s;
+            mysrc[u] = s;
+            int32_t id;
+            if constexpr (G == 1) {
+                id = (s >= 0) ? __builtin_amdgcn_readlane(my_id, s) : 0;
+            } else {
+                id = __shfl(my_id, s >= 0 ? s : 0);
+            }
+            const float4 *row = reinterpret_cast<const float4 *>(vectors + (int64_t)id * dim);
+#pragma unroll
+            for (int i = 0; i < CPL; ++i) {
+                if (s >= 0 && cvalid[i]) r[u][i] = row[lig + LPR * i];
+                else r[u][i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int i = 0; i < CPL; ++i) {
+                acc = __builtin_fmaf(r[u][i].x, q[i].x, acc);
+                acc = __builtin_fmaf(r[u][i].y, q[i].y, acc);
+                acc = __builtin_fmaf(r[u][i].z, q[i].z, acc);
+                acc = __builtin_fmaf(r[u][i].w, q[i].w, acc);
+            }
+#pragma unroll
+            for (int h = LPR / 2; h >= 1; h >>= 1) acc = acc + __shfl_xor(acc, h);
+            if (lig == 0 && mysrc[u] >= 0) out_d[mysrc[u]] = clamp_distance(acc);
+        }
+    }
+}
+
+// Any dimension, any alignment: scalar loads, same summation order.
+__device__ __forceinline__ void wave_distances_generic(const float *__restrict__ q_row,
+                                                       const float *__restrict__ vectors, int dim,
+                                                       int nchunks, int32_t my_id, bool ok,
+                                                       float *__restrict__ out_d) {
+    const int lane = threadIdx.x & (kWave - 1);
+    uint64_t mask = __ballot(ok);
+    while (mask) {
+        int s = __builtin_ctzll(mask);
+        mask &= mask - 1;
+        int32_t id = __builtin_amdgcn_readlane(my_id, s);
+        const float *row = vectors + (int64_t)id * dim;
+        float acc = 0.0f;
+        for (int c = lane; c < nchunks; c += kWave) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                int i = 4 * c + j;
+                if (i < dim) acc = __builtin_fmaf(row[i], q_row[i], acc);
+            }
+        }
+#pragma unroll
+        for (int h = kWave / 2; h >= 1; h >>= 1) acc = acc + __shfl_xor(acc, h);
+        if (lane == 0) out_d[s] = clamp_distance(acc);
+    }
+}
+
+struct ExpandArgs {
+    const float *queries;
+    const float *vectors;
+    const int32_t *ids;    // direct mode: [n_rows, m] candidate ids
+    const int32_t *visit;  // visit mode: [n_rows, n_visit] node ids (else null)
+    const int32_t *beams;  // visit mode: [n_nodes, width]
+    int32_t *idx_out;      // may be null in direct mode
+    float *dist_out;
+    BeamCtrl *ctrl;        // beam-search loop only (else null): batch-wide loop state
+    int iter;              //   iteration number, from 1
+    int readahead;         //   speculative_readahead
+    int seen_cols;         //   columns of the visited list
+    int visit_stride;      // row stride of `visit` in elements
+    int64_t n_rows;
+    int64_t n_vectors;
+    int64_t n_nodes;
+    int dim;
+    int nchunks;
+    int n_visit;
+    int width;
+    int m;     // candidates per row
+    int cw;    // candidates per wavefront (<= 64)
+    int parts; // workgroups per row
+};
+
+// blockIdx -> (row, part) so that all workgroups of one row, and the same rows
+// from one launch to the next, land on the same XCD (workgroups are dealt to
+// the 8 XCDs round-robin): the query row and neighbour-table rows then hit
+// that XCD's L2.
+__device__ __forceinline__ bool map_block(const ExpandArgs &a, int64_t &row, int &part) {
+    int64_t bid = blockIdx.x;
+    int xcd = (int)(bid & 7);
+    int64_t j = bid >> 3;
+    row = (j / a.parts) * 8 + xcd;
+    part = (int)(j % a.parts);
+    return row < a.n_rows;
+}
+
+template <int CPL, int LPR, int U, bool GENERIC>
+__global__ __launch_bounds__(256) void expand_kernel(ExpandArgs a) {
+    int gate = 0;
+    if (a.ctrl) {
+        gate = beam_gate(a.ctrl, a.iter, a.readahead, a.seen_cols, blockIdx.x == 0 && threadIdx.x == 0);
+        if (gate == 2) return;
+    }
+    int64_t row;
+    int part;
+    if (!map_block(a, row, part)) return;
+    const int wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int c0 = (part * 4 + wave) * a.cw;
+    if (c0 >= a.m) return;
+    const int n = min(a.cw, a.m - c0);
+    const bool has = lane < n;
+    const int slot = c0 + lane;
+
+    int32_t id = VL_MAXINT;
+    if (has) {
+        if (a.visit) {
+            int s = slot / a.width, k = slot - s * a.width;
+            int32_t node = gate ? VL_MAXINT : a.visit[row * a.visit_stride + s];
+            if (node != VL_MAXINT && (uint32_t)node < (uint64_t)a.n_nodes)
+                id = a.beams[(int64_t)node * a.width + k];
+        } else {
+            id = a.ids[row * a.m + slot];
+        }
+    }
+    const bool ok = has && id != VL_MAXINT && id >= 0 && (int64_t)id < a.n_vectors;
+    float *out_d = a.dist_out + row * a.m + c0;
+    if (has) {
+        if (a.idx_out) a.idx_out[row * a.m + slot] = ok ? id : VL_MAXINT;
+        if (!ok) out_d[lane] = VL_MAXFLOAT;
+    }
+    const float *q_row = a.queries + row * a.dim;
+    if constexpr (GENERIC)
+        wave_distances_generic(q_row, a.vectors, a.dim, a.nchunks, id, ok, out_d);
+    else
+        wave_distances<CPL, LPR, U>(q_row, a.vectors, a.dim, a.nchunks, id, ok, out_d);
+}
+
+template <int CPL, int LPR, int U>
+void launch_fast(const ExpandArgs &a, dim3 grid, hipStream_t st) {
+    hipLaunchKernelGGL((expand_kernel<CPL, LPR, U, false>), grid, dim3(256), 0, st, a);
+}
+
+}  // namespace
+
+// Host-side launcher shared by the C entry points and the beam-search loop.
+int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors, int64_t n_vectors,
+                     int64_t dim, const int32_t *ids, const int32_t *visit, int64_t n_visit,
+                     const int32_t *beams, int64_t n_nodes, int64_t width, int64_t m,
+                     int32_t *idx_out, float *dist_out, BeamCtrl *ctrl, int iter, int readahead,
+                     int seen_cols, int64_t visit_stride, hipStream_t st) {
+    if (n_rows == 0 || m == 0) return VL_OK;
+    VL_REQUIRE(dim >= 1 && dim <= (1 << 24), "dim %lld out of range", (long long)dim);
+    VL_REQUIRE(m <= (1 << 24), "row of %lld candidates is too wide", (long long)m);
+    ExpandArgs a;
+    a.queries = queries; a.vectors = vectors; a.ids = ids; a.visit = visit; a.beams = beams;
+    a.idx_out = idx_out; a.dist_out = dist_out;
+    a.ctrl = ctrl; a.iter = iter; a.readahead = readahead; a.seen_cols = seen_cols;
+    a.visit_stride = (int)visit_stride;
+    a.n_rows = n_rows; a.n_vectors = n_vectors; a.n_nodes = n_nodes;
+    a.dim = (int)dim; a.nchunks = (int)((dim + 3) / 4);
+    a.n_visit = (int)n_visit; a.width = (int)width; a.m = (int)m;
+
+    const bool aligned = (dim % 4 == 0) && (((uintptr_t)queries | (uintptr_t)vectors) % 16 == 0);
+    const int nchunks = a.nchunks;
+    // candidates per wavefront: enough to amortise the query load, few enough
+    // that one row's candidates spread over several wavefronts
+    a.cw = nchunks <= 64 ? 64 : 32;
+    if (m < a.cw * 4) a.cw = (int)((m + 3) / 4 < 8 ? 8 : (m + 3) / 4);
+    if (a.cw > 64) a.cw = 64;
+    a.parts = (int)((m + 4 * a.cw - 1) / (4 * a.cw));
+    int64_t row_groups = (n_rows + 7) / 8;
+    int64_t blocks = row_groups * 8 * a.parts;
+    VL_REQUIRE(blocks < (1ll << 31), "launch of %lld workgroups is too large", (long long)blocks);
+    dim3 grid((unsigned)blocks);
+
+    if (!aligned || nchunks > 512) {
+        hipLaunchKernelGGL((expand_kernel<1, 64, 1, true>), grid, dim3(256), 0, st, a);
+    } else if (nchunks <= 16) launch_fast<1, 16, 8>(a, grid, st);
+    else if (nchunks <= 32) launch_fast<1, 32, 8>(a, grid, st);
+    else if (nchunks <= 64) launch_fast<1, 64, 8>(a, grid, st);
+    else if (nchunks <= 128) launch_fast<2, 64, 8>(a, grid, st);
+    else if (nchunks <= 192) launch_fast<3, 64, 4>(a, grid, st);
+    else if (nchunks <= 256) launch_fast<4, 64, 4>(a, grid, st);
+    else if (nchunks <= 320) launch_fast<5, 64, 2>(a, grid, st);
+    else if (nchunks <= 384) launch_fast<6, 64, 2>(a, grid, st);
+    else if (nchunks <= 448) launch_fast<7, 64, 2>(a, grid, st);
+    else launch_fast<8, 64, 2>(a, grid, st);
+    VL_LAUNCH_CHECK("expand_kernel");
+    return VL_OK;
+}
+
+VL_EXPORT int vl_gather_distances(const float *queries, int64_t n_rows, const float *vectors,
+                                  int64_t n_vectors, int64_t dim, const int32_t *ids,
+                                  int64_t width, float *out, void *stream) {
+    VL_REQUIRE(n_rows >= 0 && width >= 0 && n_vectors >= 0, "negative size");
+    if (n_rows == 0 || width == 0) return VL_OK;
+    VL_REQUIRE(queries && vectors && ids && out, "null pointer");
+    return vl_launch_expand(queries, n_rows, vectors, n_vectors, dim, ids, nullptr, 0, nullptr, 0,
+                            width, width, nullptr, out, nullptr, 0, 1, 0, 0, (hipStream_t)stream);
+}
+
+VL_EXPORT int vl_search_from_seeds(const float *queries, int64_t n_rows, int64_t dim,
+                                   const int32_t *visit, int64_t n_visit, const int32_t *beams,
+                                   int64_t n_nodes, int64_t width, const float *vectors,
+                                   int64_t n_vectors, int32_t *idx_out, float *dist_out,
+                                   void *stream) {
+    VL_REQUIRE(n_rows >= 0 && n_visit >= 0 && width >= 0, "negative size");
+    if (n_rows == 0 || n_visit == 0 || width == 0) return VL_OK;
+    VL_REQUIRE(queries && visit && beams && vectors && idx_out && dist_out, "null pointer");
+    return vl_launch_expand(queries, n_rows, vectors, n_vectors, dim, nullptr, visit, n_visit, beams,
+                            n_nodes, width, n_visit * width, idx_out, dist_out, nullptr, 0, 1, 0, n_visit,
+                            (hipStream_t)stream);
+}

@@ -1,0 +1,300 @@
+"""Graph build and beam search drivers (reference: vectorlink_gpu/ann.py).
+
+Same names, arguments and control flow as the reference; the device work goes
+to libvlgpu.so.  Differences are stated where they occur.
+"""
+from __future__ import annotations
+
+import ctypes
+import time
+from typing import Dict, Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from . import _native as nv
+from .constants import DEVICE, MAXFLOAT, MAXINT
+from .kernels import calculate_distances, gather_distances, prune_, search_from_seeds
+from .log import log_time
+from .queue import Queue
+from .utils import add_new_to_seen_, generate_circulant_beams, generate_queue_circulants, primes
+
+
+def _beam_params(batch: int, dim: int, n_vectors: int, width: int, queue: Queue, config: Dict,
+                 excl_cols: int) -> nv.BeamParams:
+    return nv.BeamParams(
+        n_rows=batch, dim=dim, n_vectors=n_vectors, width=width, queue_capacity=queue.indices.size(1),
+        queue_length=queue.length, beam_size=config["beam_size"],
+        parallel_visit_count=config["parallel_visit_count"], visit_queue_factor=config["visit_queue_factor"],
+        exclude_factor=config["exclude_factor"], speculative_readahead=config["speculative_readahead"],
+        excl_cols=excl_cols)
+
+
+_WORKSPACES: Dict[str, Tensor] = {}
+
+
+def _workspace(nbytes: int, device) -> Tensor:
+    """One growing scratch tensor per device, owned by torch's allocator."""
+    key = str(device)
+    ws = _WORKSPACES.get(key)
+    if ws is None or ws.numel() < nbytes:
+        _WORKSPACES[key] = ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+    return ws
+
+
+def closest_vectors_stepwise(query_vecs: Tensor, search_queue: Queue, vectors: Tensor, beams: Tensor, config: Dict,
+                             exclude: Optional[Tensor] = None) -> int:
+    """The loop of ann.py:38-93 statement by statement on the single-purpose
+    kernels (one launch and, for the visited list, one host sync per step).
+    Same result as closest_vectors; kept for checking the fused loop."""
+    (_, beam_size) = beams.size()
+    extra_capacity = beam_size * config["parallel_visit_count"]
+    (batch_size, _) = search_queue.size()
+    visit_queue_len = config["visit_queue_factor"] * config["beam_size"]
+    capacity = visit_queue_len + extra_capacity
+    device = vectors.device
+    visit_queue = Queue(batch_size, visit_queue_len, capacity, device=device)
+    visit_queue.initialize_from_queue(search_queue)
+    exclude_len = config["exclude_factor"] * visit_queue_len
+    seen = torch.full((batch_size, exclude_len), MAXINT, dtype=torch.int32, device=device)
+
+    progressing = True
+    count = 0
+    while progressing:
+        count += 1
+        checking_output = (count % config["speculative_readahead"]) == 0
+        neighbors_to_visit = visit_queue.pop_n_ids(config["parallel_visit_count"])
+        (indexes_of_comparisons, distances_of_comparisons) = search_from_seeds(
+            query_vecs, neighbors_to_visit, beams, vectors)
+        did_something = search_queue.insert(indexes_of_comparisons, distances_of_comparisons, exclude=exclude,
+                                            output_update=checking_output)
+        if seen is not None:
+            seen = add_new_to_seen_(seen, neighbors_to_visit)
+        if seen is not None:
+            visit_queue.insert(indexes_of_comparisons, distances_of_comparisons, exclude=seen)
+        if checking_output:
+            progressing = bool(torch.any(did_something))
+    return count
+
+
+@log_time
+def closest_vectors(query_vecs: Tensor, search_queue: Queue, vectors: Tensor, beams: Tensor, config: Dict,
+                    exclude: Optional[Tensor] = None) -> int:
+    """reference ann.py:38-93.  Updates search_queue in place; returns the
+    number of iterations run (the reference returns True).  Rows are exact on
+    [:, :search_queue.length]; the slots beyond are unspecified."""
+    assert query_vecs.dtype == torch.float32 and vectors.dtype == torch.float32 and beams.dtype == torch.int32
+    nv.require_gpu(query_vecs, vectors, beams, search_queue.indices, exclude)
+    query_vecs = query_vecs.contiguous()
+    assert vectors.is_contiguous() and beams.is_contiguous()
+    assert search_queue.indices.is_contiguous() and search_queue.distances.is_contiguous()
+    (batch, dim) = query_vecs.size()
+    assert search_queue.indices.size(0) == batch and vectors.size(1) == dim and beams.size(0) == vectors.size(0)
+    excl = None
+    if exclude is not None:
+        assert exclude.dtype == torch.int32 and exclude.size(0) == batch
+        excl = exclude.contiguous()
+    p = _beam_params(batch, dim, vectors.size(0), beams.size(1), search_queue, config,
+                     0 if excl is None else excl.size(1))
+    need = nv.check(nv.lib().vl_beam_workspace_bytes(ctypes.byref(p)))
+    ws = _workspace(need, vectors.device)
+    iterations = nv.check(nv.lib().vl_closest_vectors(
+        ctypes.byref(p), nv.ptr(query_vecs), nv.ptr(vectors), nv.ptr(beams), nv.ptr(search_queue.indices),
+        nv.ptr(search_queue.distances), nv.ptr(excl), nv.ptr(ws), ws.numel(), nv.stream()))
+    return iterations
+
+
+def excluding_self(start: int, end: int, queue_length: int = 0, device=DEVICE) -> Tensor:
+    """reference ann.py:315-320: one exclusion per row, the row's own id"""
+    return torch.arange(start, end, dtype=torch.int32, device=device).unsqueeze(1)
+
+
+def generate_ann(vectors: Tensor, config: Dict, stale_distances: bool = False) -> Tuple[Tensor, Tensor]:
+    """reference ann.py:109-193.
+
+    The reference seeds every optimisation loop with the distances of the
+    initial circulant graph and returns those too (ann.py:145-147,172,190-193),
+    so from the second loop on ids and distances no longer belong together.
+    Here the distances travel with their ids; stale_distances=True restores the
+    reference's behaviour (and then uses the step-by-step loop, because the
+    fused loop relies on an id always carrying the same distance)."""
+    (num_vecs, _) = vectors.size()
+    device = vectors.device
+    beam_size = config["beam_size"]
+    queue_length = beam_size * config["beam_queue_factor"]
+    neighbor_primes = primes(queue_length, device)
+    beams = generate_circulant_beams(num_vecs, neighbor_primes)
+    beam_distances = calculate_distances(vectors, beams)
+    distances = beam_distances
+    remaining_capacity = queue_length * config["parallel_visit_count"]
+    batch_size = config["batch_size"]
+    search = closest_vectors_stepwise if stale_distances else closest_vectors
+
+    for _ in range(0, config["optimization_loops"]):
+        next_beams = torch.empty_like(beams)
+        next_beam_distances = torch.empty_like(beam_distances)
+        for start in range(0, num_vecs, batch_size):
+            end = min(start + batch_size, num_vecs)
+            exclude = excluding_self(start, end, queue_length, device)
+            queue = Queue(end - start, queue_length, queue_length + remaining_capacity, device=device)
+            seed_distances = beam_distances if stale_distances else distances
+            queue.insert(beams.narrow(0, start, end - start), seed_distances.narrow(0, start, end - start))
+            search(vectors[start:end], queue, vectors, beams, config, exclude)
+            next_beams.narrow(0, start, end - start).copy_(queue.indices.narrow(1, 0, queue_length))
+            next_beam_distances.narrow(0, start, end - start).copy_(queue.distances.narrow(1, 0, queue_length))
+
+        if config["prune"]:
+            (beams, distances) = prune_(next_beams, next_beam_distances)
+        else:
+            (beams, distances) = (next_beams, next_beam_distances)
+
+        prefix = min(num_vecs, 1000)
+        (_, recall) = ann_calculate_recall(vectors, beams.narrow_copy(1, 0, beam_size), config,
+                                           sample=vectors[:prefix])
+        if recall == 1.0:
+            break
+    out_distances = beam_distances if stale_distances else distances
+    return (beams.narrow_copy(1, 0, beam_size), out_distances.narrow_copy(1, 0, beam_size))
+
+
+def initial_queue(vectors: Tensor, config: Dict) -> Queue:
+    """reference ann.py:196-208"""
+    queue_size = config["recall_search_queue_factor"] * config["beam_size"]
+    (batch_size, _) = vectors.size()
+    extra_capacity = max(queue_size, config["parallel_visit_count"] * config["beam_size"])
+    queue = Queue(batch_size, queue_size, queue_size + extra_capacity, device=vectors.device)
+    p = primes(queue_size, vectors.device)
+    initial_queue_indices = generate_circulant_beams(batch_size, p)
+    d = calculate_distances(vectors, initial_queue_indices)
+    queue.insert(initial_queue_indices, d)
+    return queue
+
+
+def query_cosine_distances(query_vectors: Tensor, vectors: Tensor, ids: Tensor) -> Tensor:
+    """d[b, j] = clamp((1 - <query[b], vectors[ids[b, j]]>) / 2, 0, 1).
+
+    The reference's version (ann.py:211-214) multiplies [B, D] by a gathered
+    [B, Q, D] tensor, which only broadcasts for one query, and leaves out the
+    clamp; this one evaluates the seeds with the kernel every other distance
+    uses, so a seed found again during the search carries identical bits."""
+    return gather_distances(query_vectors, vectors, ids)
+
+
+def initial_search_queue(vectors: Tensor, query_vectors: Tensor, config: Dict,
+                         queue_size: Optional[int] = None) -> Queue:
+    """reference ann.py:217-232; queue_size overrides recall_search_queue_factor * beam_size"""
+    if queue_size is None:
+        queue_size = config["recall_search_queue_factor"] * config["beam_size"]
+    (batch_size, _) = query_vectors.size()
+    extra_capacity = max(queue_size, config["parallel_visit_count"] * config["beam_size"])
+    queue = Queue(batch_size, queue_size, queue_size + extra_capacity, device=vectors.device)
+    p = primes(queue_size, vectors.device)
+    (vector_count, _) = vectors.size()
+    initial_queue_indices = generate_queue_circulants(batch_size, vector_count, p)
+    d = query_cosine_distances(query_vectors, vectors, initial_queue_indices)
+    queue.insert(initial_queue_indices, d)
+    return queue
+
+
+def ann_calculate_recall(vectors: Tensor, beams: Tensor, config: Dict, sample: Optional[Tensor] = None,
+                         verbose: bool = False):
+    """reference ann.py:235-259: share of sample rows whose best hit is themselves"""
+    if sample is None:
+        sample = vectors
+    (sample_size, _) = sample.size()
+    queue = initial_queue(sample.contiguous(), config)
+    closest_vectors(sample, queue, vectors, beams.contiguous(), config)
+    expected = torch.arange(sample_size, device=vectors.device)
+    actual = queue.indices.t()[0]
+    found = (expected == actual).sum().item()
+    if verbose:
+        print(f"found: {found} / {sample_size}")
+        print(f"recall: {found / sample_size}")
+    return (found, found / sample_size)
+
+
+class ANN:
+    """reference ann.py:356-489"""
+
+    def __init__(
+        self,
+        vectors: Tensor,
+        prune: bool = True,
+        beam_size: int = 24,
+        parallel_visit_count: int = 4,
+        beam_queue_factor: int = 3,
+        visit_queue_factor: int = 3,
+        exclude_factor: int = 5,
+        optimization_loops: int = 3,
+        batch_size: int = 10_000,
+        recall_search_queue_factor: int = 3,
+        speculative_readahead: int = 5,
+        beams: Optional[Tensor] = None,
+        distances: Optional[Tensor] = None,
+    ):
+        assert vectors.dim() == 2 and vectors.dtype == torch.float32
+        (count, dim) = vectors.size()
+        self.configuration: Dict = {
+            "prune": prune,
+            "beam_size": beam_size,
+            "parallel_visit_count": parallel_visit_count,
+            "beam_queue_factor": beam_queue_factor,
+            "visit_queue_factor": visit_queue_factor,
+            "exclude_factor": exclude_factor,
+            "optimization_loops": optimization_loops,
+            "batch_size": batch_size,
+            "recall_search_queue_factor": recall_search_queue_factor,
+            "speculative_readahead": speculative_readahead,
+        }
+        if not vectors.is_cuda:
+            vectors = vectors.to(DEVICE)
+        self.vectors = vectors.contiguous()
+        wall_start = time.time()
+        if beams is not None:
+            self.beams = beams.to(self.vectors.device).contiguous()
+            if distances is None:
+                self.distances = calculate_distances(self.vectors, self.beams)
+            else:
+                self.distances = distances.to(self.vectors.device).contiguous()
+        else:
+            (self.beams, self.distances) = generate_ann(self.vectors, self.configuration)
+        torch.cuda.synchronize(self.vectors.device)
+        wall_end = time.time()
+        self.log = self.configuration.copy()
+        self.log["total_time"] = wall_end - wall_start
+        self.log["vector_count"] = count
+        self.log["vector_dimension"] = dim
+
+    def recall(self, sample_size: int = 1000) -> Tuple[float, float]:
+        """reference ann.py:456-464"""
+        (count, _) = self.vectors.size()
+        sample_size = min(sample_size, count)
+        sample = self.vectors[0:sample_size]
+        return ann_calculate_recall(self.vectors, self.beams, self.configuration, sample)
+
+    def clusters(self):
+        """reference ann.py:466-467 (a stub there as well)"""
+        return None
+
+    def search(self, query: Tensor, queue_size: Optional[int] = None) -> Queue:
+        """reference ann.py:469-477: takes a batch of query vectors, returns the
+        search Queue; the answer is queue.indices[:, :k] / queue.distances[:, :k].
+        queue_size overrides the configured search-queue length."""
+        assert query.dim() == 2 and query.dtype == torch.float32
+        if not query.is_cuda:
+            query = query.to(self.vectors.device)
+        query = query.contiguous()
+        search_queue = initial_search_queue(self.vectors, query, self.configuration, queue_size)
+        closest_vectors(query, search_queue, self.vectors, self.beams, self.configuration, None)
+        return search_queue
+
+    def dump_logs(self) -> Dict:
+        """reference ann.py:479-489 without the nvidia-smi / git shell-outs"""
+        from . import log as _log
+
+        out = self.log.copy()
+        out["closest_vectors_batch_time"] = _log.CLOSEST_VECTORS_BATCH_TIME
+        out["gpu_arch"] = torch.cuda.get_device_name(self.vectors.device)
+        (_, recall) = self.recall()
+        out["recall"] = recall
+        return out

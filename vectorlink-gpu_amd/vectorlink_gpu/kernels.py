@@ -1,0 +1,154 @@
+"""Launchers with the names and signatures of the reference's
+vectorlink_gpu/kernels.py; every body is a call into libvlgpu.so (hand-written
+HIP for gfx950) on torch's current stream."""
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from . import _native as nv
+from .constants import MAXFLOAT, MAXINT
+from .log import log_time
+
+
+def _check_ids(t: Tensor, name: str):
+    assert t.dtype == torch.int32, f"{name} must be int32"
+    assert t.is_contiguous(), f"{name} must be contiguous"
+
+
+def _check_f32(t: Tensor, name: str):
+    assert t.dtype == torch.float32, f"{name} must be float32"
+    assert t.is_contiguous(), f"{name} must be contiguous"
+
+
+def gather_distances(queries: Tensor, vectors: Tensor, ids: Tensor, out: Optional[Tensor] = None) -> Tensor:
+    """out[r, j] = cosine distance of queries[r] and vectors[ids[r, j]] (MAXFLOAT for MAXINT ids)."""
+    _check_f32(queries, "queries")
+    _check_f32(vectors, "vectors")
+    _check_ids(ids, "ids")
+    nv.require_gpu(queries, vectors, ids)
+    (rows, width) = ids.size()
+    assert queries.size(0) == rows and queries.size(1) == vectors.size(1)
+    if out is None:
+        out = torch.empty((rows, width), dtype=torch.float32, device=ids.device)
+    else:
+        _check_f32(out, "out")
+        assert out.size() == ids.size()
+    nv.check(nv.lib().vl_gather_distances(nv.ptr(queries), rows, nv.ptr(vectors), vectors.size(0), vectors.size(1),
+                                          nv.ptr(ids), width, nv.ptr(out), nv.stream()))
+    return out
+
+
+@log_time
+def calculate_distances(vectors: Tensor, beams: Tensor, distances_out: Optional[Tensor] = None) -> Tensor:
+    """reference kernels.py:174-201"""
+    _check_f32(vectors, "vectors")
+    _check_ids(beams, "beams")
+    (vector_count, _) = vectors.size()
+    (batches, _) = beams.size()
+    assert batches == vector_count  # kernels.py:186
+    return gather_distances(vectors, vectors, beams, distances_out)
+
+
+def search_from_seeds(query_vecs: Tensor, neighbors_to_visit: Tensor, beams: Tensor,
+                      vectors: Tensor) -> Tuple[Tensor, Tensor]:
+    """reference kernels.py:260-311"""
+    _check_f32(query_vecs, "query_vecs")
+    _check_ids(neighbors_to_visit, "neighbors_to_visit")
+    _check_ids(beams, "beams")
+    _check_f32(vectors, "vectors")
+    nv.require_gpu(query_vecs, neighbors_to_visit, beams, vectors)
+    (batch_size, visit_length) = neighbors_to_visit.size()
+    (node_count, beam_size) = beams.size()
+    (vector_count, dim) = vectors.size()
+    assert query_vecs.size(0) == batch_size and query_vecs.size(1) == dim
+    index_out = torch.empty((batch_size, visit_length * beam_size), dtype=torch.int32, device=vectors.device)
+    distance_out = torch.empty((batch_size, visit_length * beam_size), dtype=torch.float32, device=vectors.device)
+    nv.check(nv.lib().vl_search_from_seeds(nv.ptr(query_vecs), batch_size, dim, nv.ptr(neighbors_to_visit),
+                                           visit_length, nv.ptr(beams), node_count, beam_size, nv.ptr(vectors),
+                                           vector_count, nv.ptr(index_out), nv.ptr(distance_out), nv.stream()))
+    return (index_out, distance_out)
+
+
+def dedup_tensor_(ids: Tensor):
+    """reference kernels.py:370-380 (in place)"""
+    _check_ids(ids, "ids")
+    nv.require_gpu(ids)
+    nv.check(nv.lib().vl_dedup_ids(nv.ptr(ids), ids.size(0), ids.size(1), nv.stream()))
+
+
+def dedup_tensor_pair_(ids: Tensor, distances: Tensor):
+    """reference kernels.py:383-397 (in place; assumes sorted rows)"""
+    _check_ids(ids, "ids")
+    _check_f32(distances, "distances")
+    assert ids.size() == distances.size()
+    nv.require_gpu(ids, distances)
+    nv.check(nv.lib().vl_dedup_pairs(nv.ptr(ids), nv.ptr(distances), ids.size(0), ids.size(1), nv.stream()))
+
+
+def punchout_duplicates_(ids: Tensor, distances: Tensor):
+    """reference kernels.py:400-406; works in place and returns the same tensors"""
+    _check_ids(ids, "ids")
+    _check_f32(distances, "distances")
+    assert ids.size() == distances.size()
+    nv.require_gpu(ids, distances)
+    nv.check(nv.lib().vl_punchout_duplicates(nv.ptr(ids), nv.ptr(distances), ids.size(0), ids.size(1), nv.stream()))
+    return (ids, distances)
+
+
+def prune_(beams: Tensor, distances: Tensor):
+    """reference kernels.py:441-468.  Decisions are taken from the tables as
+    passed in and the result is returned in new tensors; the inputs are left
+    untouched (the reference marks them in place while other blocks read)."""
+    _check_ids(beams, "beams")
+    _check_f32(distances, "distances")
+    assert beams.size() == distances.size()
+    nv.require_gpu(beams, distances)
+    out_b = torch.empty_like(beams)
+    out_d = torch.empty_like(distances)
+    nv.check(nv.lib().vl_prune(nv.ptr(beams), nv.ptr(distances), beams.size(0), beams.size(1), nv.ptr(out_b),
+                               nv.ptr(out_d), nv.stream()))
+    return (out_b, out_d)
+
+
+def punchout_excluded_(indices: Tensor, distances: Tensor, exclusions: Tensor):
+    """reference kernels.py:491-501; indices/distances may be column slices of a wider tensor"""
+    assert indices.dtype == torch.int32 and distances.dtype == torch.float32 and exclusions.dtype == torch.int32
+    assert indices.dim() == 2 and indices.size() == distances.size()
+    assert indices.stride(1) == 1 and distances.stride(1) == 1 and exclusions.stride(1) == 1
+    (batch_size, queue_size) = indices.size()
+    (batch_size2, exclusion_size) = exclusions.size()
+    assert batch_size == batch_size2
+    nv.require_gpu(indices, distances, exclusions)
+    nv.check(nv.lib().vl_punchout_excluded(nv.ptr(indices), nv.ptr(distances), batch_size, queue_size,
+                                           indices.stride(0) if batch_size > 1 else queue_size,
+                                           distances.stride(0) if batch_size > 1 else queue_size,
+                                           nv.ptr(exclusions), exclusion_size,
+                                           exclusions.stride(0) if batch_size > 1 else exclusion_size, nv.stream()))
+
+
+def index_by_tensor(a: Tensor, b: Tensor) -> Tensor:
+    """reference kernels.py:554-559: out[r, c] = a[r, b[r, c]]"""
+    assert a.dim() == 2 and a.size() == b.size() and a.element_size() == 4
+    nv.require_gpu(a, b)
+    a = a.contiguous()
+    b = b.contiguous().to(torch.int64)
+    out = torch.empty_like(a)
+    nv.check(nv.lib().vl_index_by_tensor(nv.ptr(a), nv.ptr(b), nv.ptr(out), a.size(0), a.size(1), nv.stream()))
+    return out
+
+
+def index_sort_(ids: Tensor, distances: Tensor):
+    """order rows by (distance, id) in place (reference utils.py:44-53)"""
+    _check_ids(ids, "ids")
+    _check_f32(distances, "distances")
+    nv.require_gpu(ids, distances)
+    nv.check(nv.lib().vl_index_sort(nv.ptr(ids), nv.ptr(distances), ids.size(0), ids.size(1), nv.stream()))
+
+
+def queue_sort_(ids: Tensor, distances: Tensor):
+    """reference queue.py:15-18, in place"""
+    _check_ids(ids, "ids")
+    _check_f32(distances, "distances")
+    nv.require_gpu(ids, distances)
+    nv.check(nv.lib().vl_queue_sort(nv.ptr(ids), nv.ptr(distances), ids.size(0), ids.size(1), nv.stream()))
