@@ -165,6 +165,14 @@ int64_t vl_closest_vectors(const vl_beam_params *p,
                            void *workspace, int64_t workspace_bytes,
                            void *stream);
 
+/* Per-kernel timing of vl_closest_vectors (no counterpart in the reference,
+ * whose log.py:7-17 times whole calls): with enable != 0 every expand / merge
+ * launch is bracketed by HIP events on the caller's stream.  out (7 doubles,
+ * may be NULL) receives the sums since the last reset: expand ms, merge ms,
+ * expand launches, merge launches, candidate rows fetched, query rows,
+ * iterations.  Not thread safe. */
+int vl_beam_profile(int enable, int reset, double *out);
+
 /* ---- pruning (kernels.py:441-468 prune_) ------------------------------ */
 
 /* For every x and slot j: y = beams[x,j], z = beams[y,0]; if z occurs in row
@@ -174,6 +182,18 @@ int64_t vl_closest_vectors(const vl_beam_params *p,
  * while other blocks read); results go to the *_out tables. */
 int vl_prune(const int32_t *beams, const float *dists, int64_t n, int64_t width,
              int32_t *beams_out, float *dists_out, void *stream);
+
+/* ---- exact k nearest neighbours on dense fp32 MFMA tiles -------------- */
+/* No counterpart in the reference (its recall is self-recall@1 only,
+ * ann.py:235-259); used for ground truth recall@k.  ids_out/dists_out are
+ * [n_queries, k], ordered by (distance, id).  k <= 16, dim % 4 == 0,
+ * pointers 16-byte aligned.  Distances come from MFMA accumulation, so they
+ * agree with the gathered-distance kernels to ~1e-7, not bit for bit. */
+int64_t vl_knn_workspace_bytes(int64_t n_queries, int64_t n_vectors, int64_t dim, int64_t k);
+int vl_knn_exact(const float *queries, int64_t n_queries,
+                 const float *vectors, int64_t n_vectors, int64_t dim, int64_t k,
+                 int32_t *ids_out, float *dists_out,
+                 void *workspace, int64_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

@@ -368,3 +368,30 @@ def test_generate_ann_stale_distance_mode():
     wb, wd = orc.generate_ann(v, c, stale_distances=True)
     gb, gd = generate_ann(dev(v), c, stale_distances=True)
     assert np.array_equal(host(gb), wb) and np.array_equal(bits(host(gd)), bits(wd))
+
+
+# ---------------------------------------------------------------- exact kNN tiles
+@pytest.mark.parametrize("n,dim,nq,k", [(5000, 128, 300, 10), (3000, 768, 129, 10), (1000, 20, 7, 16), (700, 36, 260, 1),
+                                        (130, 8, 5, 10), (20000, 64, 64, 10)])
+def test_knn_exact(n, dim, nq, k):
+    say(f"knn_exact n={n} dim={dim} nq={nq} k={k}")
+    from vectorlink_gpu.kernels import knn_exact
+
+    rng = np.random.default_rng(n + dim)
+    v = unit(rng, n, dim)
+    q = unit(rng, nq, dim)
+    q[0] = v[17]  # an exact hit at distance 0
+    wi, wd = orc.knn_exact(q, v, k)
+    gi, gd = knn_exact(dev(q), dev(v), k)
+    gi, gd = host(gi), host(gd)
+    assert np.allclose(gd, wd, rtol=1e-5, atol=1e-6)
+    assert gi[0, 0] == 17
+    assert (np.diff(gd, axis=1) >= 0).all()
+    # ids agree except where two distances are closer than float32 MFMA rounding can order
+    mism = gi != wi
+    assert mism.mean() < 0.01
+    for r, c in zip(*np.nonzero(mism)):
+        d_true = (1 - float(np.dot(q[r].astype(np.float64), v[gi[r, c]]))) / 2
+        assert abs(d_true - wd[r, c]) < 2e-6
+    for r in range(nq):
+        assert len(set(gi[r].tolist())) == k

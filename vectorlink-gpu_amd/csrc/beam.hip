@@ -21,11 +21,20 @@ int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors,
                      int64_t dim, const int32_t *ids, const int32_t *visit, int64_t n_visit,
                      const int32_t *beams, int64_t n_nodes, int64_t width, int64_t m,
                      int32_t *idx_out, float *dist_out, BeamCtrl *ctrl, int iter, int readahead,
-                     int seen_cols, int64_t visit_stride, hipStream_t st);
+                     int seen_cols, int64_t visit_stride, int count_evals, hipStream_t st);
 
 namespace {
 
 constexpr int kMaxVisit = 64;  // parallel_visit_count handled by one wavefront
+
+// Optional per-kernel timing of the loop (off by default): HIP events around
+// every expand and merge launch on the caller's stream, summed per call.
+struct BeamProfile {
+    int enabled = 0;
+    double expand_ms = 0, merge_ms = 0;
+    int64_t expand_launches = 0, merge_launches = 0, evals = 0, rows = 0, iterations = 0;
+};
+BeamProfile g_prof;
 
 struct MergeArgs {
     BeamCtrl *ctrl;
@@ -76,7 +85,10 @@ __global__ __launch_bounds__(kQueueThreads) void beam_init_kernel(BeamCtrl *ctrl
         ctrl->reserved = 0;
         ctrl->first[0] = ctrl->first[1] = 0;
     }
-    if (t < 64) ctrl->changed[t] = 0;
+    if (t < 64) {
+        ctrl->changed[t] = 0;
+        ctrl->evals[t] = 0;
+    }
     if (t < n_rows) seen_count[t] = 0;
     if (t < n_rows * VL) {  // Queue.initialize_from_queue, queue.py:30-35
         int64_t r = t / VL;
@@ -330,22 +342,68 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
     VL_REQUIRE(smem <= 60 * 1024, "queues of this size need %zu bytes of LDS (limit 61440)", smem);
 
     const int R = (int)p->speculative_readahead;
+    const bool prof = g_prof.enabled != 0;
+    hipEvent_t ev[3 * 64];
+    if (prof) {
+        VL_REQUIRE(R <= 64, "profiling supports speculative_readahead up to 64");
+        for (int i = 0; i < 3 * R; ++i) VL_HIP(hipEventCreate(&ev[i]));
+    }
     int64_t t = 0;
     for (;;) {
         for (int r = 0; r < R; ++r) {
             ++t;
+            if (prof) VL_HIP(hipEventRecord(ev[3 * r], st));
             rc = vl_launch_expand(queries, p->n_rows, vectors, p->n_vectors, p->dim, nullptr, v_ids, l.Vt, beams,
-                                  p->n_vectors, p->width, l.m, cand_ids, cand_d, ctrl, (int)t, R, (int)l.E, l.VL, st);
+                                  p->n_vectors, p->width, l.m, cand_ids, cand_d, ctrl, (int)t, R, (int)l.E, l.VL,
+                                  prof ? 1 : 0, st);
             if (rc < 0) return rc;
+            if (prof) VL_HIP(hipEventRecord(ev[3 * r + 1], st));
             a.iter = (int)t;
             hipLaunchKernelGGL(beam_merge_kernel, dim3((unsigned)p->n_rows), dim3(kQueueThreads), smem, st, a);
             VL_LAUNCH_CHECK("beam_merge_kernel");
+            if (prof) VL_HIP(hipEventRecord(ev[3 * r + 2], st));
         }
         int changed = 0;
         VL_HIP(hipMemcpyAsync(&changed, &ctrl->changed[(t / R) & 63], sizeof(int), hipMemcpyDeviceToHost, st));
         VL_HIP(hipStreamSynchronize(st));
+        if (prof) {
+            for (int r = 0; r < R; ++r) {
+                float ms = 0;
+                VL_HIP(hipEventElapsedTime(&ms, ev[3 * r], ev[3 * r + 1]));
+                g_prof.expand_ms += ms;
+                VL_HIP(hipEventElapsedTime(&ms, ev[3 * r + 1], ev[3 * r + 2]));
+                g_prof.merge_ms += ms;
+            }
+            g_prof.expand_launches += R;
+            g_prof.merge_launches += R;
+        }
         if (!changed) break;  // ann.py:90-91
         VL_REQUIRE(t < (1ll << 30), "beam search did not terminate");
     }
+    if (prof) {
+        unsigned long long ev_counts[64];
+        VL_HIP(hipMemcpyAsync(ev_counts, ctrl->evals, sizeof(ev_counts), hipMemcpyDeviceToHost, st));
+        VL_HIP(hipStreamSynchronize(st));
+        for (int i = 0; i < 64; ++i) g_prof.evals += (int64_t)ev_counts[i];
+        g_prof.rows += p->n_rows;
+        g_prof.iterations += t;
+        for (int i = 0; i < 3 * R; ++i) (void)hipEventDestroy(ev[i]);
+    }
     return t;
+}
+
+// Profiling switch for vl_closest_vectors: when enabled every expand / merge
+// launch is bracketed by HIP events on the caller's stream and the fetched
+// candidate rows are counted.  out[0..6] = expand ms, merge ms, expand
+// launches, merge launches, candidate rows fetched, query rows, iterations,
+// summed since the last reset.
+VL_EXPORT int vl_beam_profile(int enable, int reset, double *out) {
+    if (out) {
+        out[0] = g_prof.expand_ms; out[1] = g_prof.merge_ms;
+        out[2] = (double)g_prof.expand_launches; out[3] = (double)g_prof.merge_launches;
+        out[4] = (double)g_prof.evals; out[5] = (double)g_prof.rows; out[6] = (double)g_prof.iterations;
+    }
+    if (reset) g_prof = BeamProfile();
+    g_prof.enabled = enable;
+    return VL_OK;
 }

@@ -14,6 +14,7 @@ struct BeamCtrl {
     int reserved;
     int first[2];
     int changed[64];
+    unsigned long long evals[64];  // profiling only: candidate rows actually fetched, striped by workgroup
 };
 
 // State of iteration t as seen by a kernel launched for it:

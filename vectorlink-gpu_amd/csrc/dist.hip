@@ -141,6 +141,7 @@ struct ExpandArgs {
     int readahead;         //   speculative_readahead
     int seen_cols;         //   columns of the visited list
     int visit_stride;      // row stride of `visit` in elements
+    int count_evals;       //   profiling: add the number of fetched rows to ctrl->evals
     int64_t n_rows;
     int64_t n_vectors;
     int64_t n_nodes;
@@ -201,6 +202,10 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs a) {
         if (a.idx_out) a.idx_out[row * a.m + slot] = ok ? id : VL_MAXINT;
         if (!ok) out_d[lane] = VL_MAXFLOAT;
     }
+    if (a.count_evals) {
+        uint64_t okm = __ballot(ok);
+        if (lane == 0 && okm) atomicAdd(&a.ctrl->evals[blockIdx.x & 63], (unsigned long long)__popcll(okm));
+    }
     const float *q_row = a.queries + row * a.dim;
     if constexpr (GENERIC)
         wave_distances_generic(q_row, a.vectors, a.dim, a.nchunks, id, ok, out_d);
@@ -220,7 +225,7 @@ int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors,
                      int64_t dim, const int32_t *ids, const int32_t *visit, int64_t n_visit,
                      const int32_t *beams, int64_t n_nodes, int64_t width, int64_t m,
                      int32_t *idx_out, float *dist_out, BeamCtrl *ctrl, int iter, int readahead,
-                     int seen_cols, int64_t visit_stride, hipStream_t st) {
+                     int seen_cols, int64_t visit_stride, int count_evals, hipStream_t st) {
     if (n_rows == 0 || m == 0) return VL_OK;
     VL_REQUIRE(dim >= 1 && dim <= (1 << 24), "dim %lld out of range", (long long)dim);
     VL_REQUIRE(m <= (1 << 24), "row of %lld candidates is too wide", (long long)m);
@@ -229,6 +234,7 @@ int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors,
     a.idx_out = idx_out; a.dist_out = dist_out;
     a.ctrl = ctrl; a.iter = iter; a.readahead = readahead; a.seen_cols = seen_cols;
     a.visit_stride = (int)visit_stride;
+    a.count_evals = ctrl ? count_evals : 0;
     a.n_rows = n_rows; a.n_vectors = n_vectors; a.n_nodes = n_nodes;
     a.dim = (int)dim; a.nchunks = (int)((dim + 3) / 4);
     a.n_visit = (int)n_visit; a.width = (int)width; a.m = (int)m;
@@ -269,7 +275,7 @@ VL_EXPORT int vl_gather_distances(const float *queries, int64_t n_rows, const fl
     if (n_rows == 0 || width == 0) return VL_OK;
     VL_REQUIRE(queries && vectors && ids && out, "null pointer");
     return vl_launch_expand(queries, n_rows, vectors, n_vectors, dim, ids, nullptr, 0, nullptr, 0,
-                            width, width, nullptr, out, nullptr, 0, 1, 0, 0, (hipStream_t)stream);
+                            width, width, nullptr, out, nullptr, 0, 1, 0, 0, 0, (hipStream_t)stream);
 }
 
 VL_EXPORT int vl_search_from_seeds(const float *queries, int64_t n_rows, int64_t dim,
@@ -281,6 +287,6 @@ VL_EXPORT int vl_search_from_seeds(const float *queries, int64_t n_rows, int64_t
     if (n_rows == 0 || n_visit == 0 || width == 0) return VL_OK;
     VL_REQUIRE(queries && visit && beams && vectors && idx_out && dist_out, "null pointer");
     return vl_launch_expand(queries, n_rows, vectors, n_vectors, dim, nullptr, visit, n_visit, beams,
-                            n_nodes, width, n_visit * width, idx_out, dist_out, nullptr, 0, 1, 0, n_visit,
+                            n_nodes, width, n_visit * width, idx_out, dist_out, nullptr, 0, 1, 0, n_visit, 0,
                             (hipStream_t)stream);
 }

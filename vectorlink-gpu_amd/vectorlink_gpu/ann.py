@@ -14,7 +14,7 @@ from torch import Tensor
 
 from . import _native as nv
 from .constants import DEVICE, MAXFLOAT, MAXINT
-from .kernels import calculate_distances, gather_distances, prune_, search_from_seeds
+from .kernels import calculate_distances, gather_distances, knn_exact, prune_, search_from_seeds
 from .log import log_time
 from .queue import Queue
 from .utils import add_new_to_seen_, generate_circulant_beams, generate_queue_circulants, primes
@@ -287,6 +287,18 @@ class ANN:
         search_queue = initial_search_queue(self.vectors, query, self.configuration, queue_size)
         closest_vectors(query, search_queue, self.vectors, self.beams, self.configuration, None)
         return search_queue
+
+    def recall_at_k(self, query: Tensor, k: int = 10, queue_size: Optional[int] = None) -> float:
+        """Share of the exact k nearest neighbours (brute force on MFMA tiles)
+        that search() returns in its first k slots.  Not in the reference,
+        whose recall() is self-recall@1."""
+        if not query.is_cuda:
+            query = query.to(self.vectors.device)
+        query = query.contiguous()
+        found = self.search(query, queue_size).indices[:, :k]
+        (truth, _) = knn_exact(query, self.vectors, k)
+        hits = (found.unsqueeze(2) == truth.unsqueeze(1)).any(dim=2).sum().item()
+        return hits / truth.numel()
 
     def dump_logs(self) -> Dict:
         """reference ann.py:479-489 without the nvidia-smi / git shell-outs"""
