@@ -1,0 +1,240 @@
+#!/usr/bin/env python3
+"""Benchmark of the ANN hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mix-1m-768]
+
+A step is one batch of 10,000 vectors taken through the beam search of the
+graph build (closest_vectors) against the current graph.  By default K is the
+whole build - every batch of every optimisation loop, with prune and the
+per-loop self-recall - so `value` is N / wall time of the build.  With a smaller
+K the first K steps are timed and `value` is the projected build rate
+(K * batch / time / optimisation_loops), flagged "partial".  Warm-up steps run
+on a throw-away 50,000-vector build and never touch the timed one.
+
+After a complete build the search leg sweeps the search-queue length, measures
+recall@10 against exact kNN (MFMA tiles) and reports QPS at the shortest queue
+reaching 0.95.  One JSON line goes to stdout.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "vectorlink-gpu_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+# Bytes moved past L2 per expand launch, from two rocprofv3 --pmc runs (FETCH_SIZE x 2.0 after calibration
+# against a 1 GiB copy, + WRITE_SIZE x 1.0); profiles/expand_kernel_mix-1m-768_hbm_traffic.txt holds the runs.
+# Workloads without a recorded counter run report null.
+TRAFFIC_BYTES_PER_LAUNCH = {"mix-1m-768": 14.87e9}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def profile_read(nv, reset=True, enable=1):
+    out = (ctypes.c_double * 7)()
+    nv.lib().vl_beam_profile(enable, 1 if reset else 0, out)
+    keys = ("expand_ms", "merge_ms", "expand_launches", "merge_launches", "evals", "rows", "iterations")
+    return dict(zip(keys, list(out)))
+
+
+def cpu_baseline(vectors_cpu, cfg, n_rows, scale, gpu_fn):
+    """Times the CPU oracle's closest_vectors on the first n_rows rows of the
+    same workload in the state the build starts from (circulant graph), checks
+    the GPU's ids for the same batch, and scales the rate to whole-build
+    vectors/s with the GPU's own ratio of first-loop time to build time.
+    Test infrastructure used as the reported CPU baseline."""
+    from oracle import oracle as orc
+
+    threads = min(16, os.cpu_count() or 1)
+    orc.set_threads(threads)
+    v = vectors_cpu.numpy()
+    n = v.shape[0]
+    ql = cfg["beam_size"] * cfg["beam_queue_factor"]
+    beams = orc.generate_circulant_beams(n, orc.primes(ql))
+    d_rows = orc.gather_distances(v[:n_rows], v, beams[:n_rows])
+    q = orc.Queue(n_rows, ql, ql + ql * cfg["parallel_visit_count"])
+    q.insert(beams[:n_rows], d_rows)
+    t0 = time.time()
+    iters = orc.closest_vectors(v[:n_rows], q, v, beams, cfg, orc.excluding_self(0, n_rows))
+    dt = time.time() - t0
+    gpu_ids, gpu_d = gpu_fn(n_rows)
+    ok = bool((q.indices[:, :ql] == gpu_ids).all() and (q.distances[:, :ql] == gpu_d).all())
+    return dict(value=n_rows / dt * scale, unit="vectors/s", cores=threads, kind="port",
+                sample=f"oracle closest_vectors on rows [0,{n_rows}) of the same workload against the initial "
+                       f"circulant graph: {iters} iterations in {dt:.1f} s = {n_rows / dt:.1f} rows/s per loop, "
+                       f"scaled by the GPU's first-loop/whole-build time ratio {scale:.3f}",
+                ids_and_distances_match_gpu=ok)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=0, help="batch steps to time (0 = the whole build)")
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="mix-1m-768")
+    ap.add_argument("--n", type=int, default=None, help="override the number of vectors")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first run one plain 1 GiB device copy (a known-size kernel to scale rocprofv3 counters by)")
+    ap.add_argument("--cpu-rows", type=int, default=768)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+
+    from vectorlink_gpu import _native as nv
+    from vectorlink_gpu import synthetic
+    from vectorlink_gpu.ann import ANN, GraphBuild
+    from vectorlink_gpu.kernels import knn_exact
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    nv.lib()  # fail loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+
+    t0 = time.time()
+    base, queries, w = synthetic.make(args.workload, n=args.n)
+    n, dim = base.shape
+    log(f"[bench] workload {args.workload}: {n} x {dim}, generated in {time.time() - t0:.1f} s")
+    kwargs = synthetic.ann_kwargs(w)
+    cfg = dict(prune=True, parallel_visit_count=4, visit_queue_factor=3, exclude_factor=5, optimization_loops=3,
+               batch_size=10_000, speculative_readahead=5, **kwargs)
+    vectors = base.to(dev)
+    qdev = queries.to(dev)
+    torch.cuda.synchronize()
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # 1 GiB read + 1 GiB written by one elementwise copy kernel
+        torch.cuda.synchronize()
+        del src, dst
+
+    # warm-up: a small separate build (kernels compiled/loaded, allocator primed)
+    if args.warmup > 0:
+        wb = GraphBuild(vectors[:50_000].contiguous(), cfg)
+        for i, _ in enumerate(wb.steps()):
+            if i + 1 >= args.warmup:
+                break
+        torch.cuda.synchronize()
+        del wb
+
+    profile_read(nv, reset=True, enable=1)
+    torch.cuda.synchronize()
+    t_start = time.time()
+    build = GraphBuild(vectors, cfg)
+    total_steps = build.batches_per_loop() * cfg["optimization_loops"]
+    want = args.steps if args.steps > 0 else total_steps
+    done = 0
+    rows_done = 0
+    for (loop, start, end, iters) in build.steps():
+        done += 1
+        rows_done += end - start
+        if done >= want:
+            break
+    torch.cuda.synchronize()
+    t_build = time.time() - t_start
+    prof = profile_read(nv, reset=True, enable=0)
+    complete = build.finished or done >= total_steps
+    loops_run = len(build.stats)
+    if complete:
+        value = n / t_build
+    else:
+        value = rows_done / t_build / cfg["optimization_loops"]
+    log(f"[bench] build: {done} steps in {t_build:.1f} s -> {value:.0f} vectors/s"
+        f"{'' if complete else ' (partial, projected)'}; loops: {build.stats}")
+
+    bytes_per_eval = 4 * dim + 12
+    # algorithmic bytes: 4*dim + 12 per candidate row actually evaluated, plus the query row
+    # (4*dim) once per (row, iteration); prof["iterations"] sums iterations over batches
+    launches = max(prof["expand_launches"], 1.0)
+    q_loads = prof["iterations"] * min(cfg["batch_size"], n) * 4.0 * dim
+    algo_bytes = prof["evals"] * bytes_per_eval + q_loads
+    achieved = algo_bytes / (prof["expand_ms"] / 1e3) / 1e9 if prof["expand_ms"] > 0 else 0.0
+    roofline = dict(bound="hbm", kernel="expand_kernel (gathered cosine distances of the beam search)",
+                    achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
+                    traffic=TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
+                    launches=int(prof["expand_launches"]), avg_launch_ms=prof["expand_ms"] / launches,
+                    algorithmic_bytes_per_launch=algo_bytes / launches,
+                    merge_avg_launch_ms=prof["merge_ms"] / max(prof["merge_launches"], 1.0))
+
+    result = {
+        "metric": "build vecs/s + search QPS @recall@10=0.95, 1M×768 fp32, 1 MI355X",
+        "value": value, "unit": "vectors/s", "n_gpus": 1, "steps": done, "warmup": args.warmup,
+        "ms_per_step": t_build * 1e3 / max(done, 1), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": args.workload, "n": n, "dim": dim, "degree": cfg["beam_size"],
+                   "build_queue": cfg["beam_size"] * cfg["beam_queue_factor"], "batch_size": cfg["batch_size"],
+                   "optimization_loops": cfg["optimization_loops"], "parallel_visit_count": 4,
+                   "seeding": "circulant (reference)", "queries": int(queries.shape[0])},
+        "partial": not complete, "build_seconds": t_build, "loops": build.stats,
+        "roofline": roofline,
+    }
+
+    if complete:
+        (beams, dists) = build.result()
+        ann = ANN(vectors, beams=beams, distances=dists, **{k: v for k, v in cfg.items()})
+        torch.cuda.synchronize()
+        t0 = time.time()
+        (truth, _) = knn_exact(qdev, vectors, 10)
+        torch.cuda.synchronize()
+        t_knn = time.time() - t0
+        flops = 2.0 * qdev.shape[0] * n * dim
+        sweep = []
+        chosen = None
+        for qs in (32, 64, 96, 128, 192, 256):
+            ann.search(qdev[:256].contiguous(), queue_size=qs)  # warm the workspace for this shape
+            torch.cuda.synchronize()
+            t0 = time.time()
+            res = ann.search(qdev, queue_size=qs)
+            torch.cuda.synchronize()
+            dt = time.time() - t0
+            found = res.indices[:, :10]
+            hits = (found.unsqueeze(2) == truth.unsqueeze(1)).any(dim=2).sum().item()
+            rec = hits / truth.numel()
+            sweep.append(dict(queue=qs, qps=qdev.shape[0] / dt, recall_at_10=rec))
+            if chosen is None and rec >= 0.95:
+                chosen = sweep[-1]
+        result["search"] = dict(sweep=sweep, at_recall_0_95=chosen, reached_0_95=chosen is not None,
+                                qps=(chosen or sweep[-1])["qps"], recall_at_10=(chosen or sweep[-1])["recall_at_10"])
+        result["exact_knn"] = dict(seconds=t_knn, tflops=flops / t_knn / 1e12, peak_tflops=157.3,
+                                   frac=flops / t_knn / 1e12 / 157.3, bound="mfma")
+        log(f"[bench] search sweep: {sweep}")
+
+    if not args.no_cpu:
+        # CPU leg: the oracle on the first rows of the same workload, first-loop state
+        def gpu_same_batch(n_rows):
+            from vectorlink_gpu.ann import closest_vectors, excluding_self
+            from vectorlink_gpu.kernels import calculate_distances
+            from vectorlink_gpu.queue import Queue
+            from vectorlink_gpu.utils import generate_circulant_beams, primes
+
+            ql = cfg["beam_size"] * cfg["beam_queue_factor"]
+            b0 = generate_circulant_beams(n, primes(ql, dev))
+            d0 = calculate_distances(vectors, b0)
+            gq = Queue(n_rows, ql, ql + ql * cfg["parallel_visit_count"], device=dev)
+            gq.insert(b0[:n_rows], d0[:n_rows])
+            closest_vectors(vectors[:n_rows], gq, vectors, b0, cfg, excluding_self(0, n_rows, device=dev))
+            return gq.indices[:, :ql].cpu().numpy(), gq.distances[:, :ql].cpu().numpy()
+
+        try:
+            scale = (build.stats[0]["seconds"] / t_build) if (complete and build.stats) else 1.0 / cfg["optimization_loops"]
+            result["cpu_baseline"] = cpu_baseline(base, cfg, min(args.cpu_rows, n), scale, gpu_same_batch)
+        except Exception as e:  # the CPU leg must never take the GPU numbers down with it
+            result["cpu_baseline"] = dict(value=None, unit="vectors/s", cores=0, kind="port", sample=f"failed: {e!r}")
+
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

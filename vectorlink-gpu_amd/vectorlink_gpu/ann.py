@@ -109,8 +109,11 @@ def excluding_self(start: int, end: int, queue_length: int = 0, device=DEVICE) -
     return torch.arange(start, end, dtype=torch.int32, device=device).unsqueeze(1)
 
 
-def generate_ann(vectors: Tensor, config: Dict, stale_distances: bool = False) -> Tuple[Tensor, Tensor]:
-    """reference ann.py:109-193.
+class GraphBuild:
+    """generate_ann (reference ann.py:109-193) as a sequence of batch steps, so a
+    caller can time or interleave them.  One step = one batch of rows taken
+    through closest_vectors against the current graph; the step that ends an
+    optimisation loop also prunes and runs the self-recall test.
 
     The reference seeds every optimisation loop with the distances of the
     initial circulant graph and returns those too (ann.py:145-147,172,190-193),
@@ -118,43 +121,85 @@ def generate_ann(vectors: Tensor, config: Dict, stale_distances: bool = False) -
     Here the distances travel with their ids; stale_distances=True restores the
     reference's behaviour (and then uses the step-by-step loop, because the
     fused loop relies on an id always carrying the same distance)."""
-    (num_vecs, _) = vectors.size()
-    device = vectors.device
-    beam_size = config["beam_size"]
-    queue_length = beam_size * config["beam_queue_factor"]
-    neighbor_primes = primes(queue_length, device)
-    beams = generate_circulant_beams(num_vecs, neighbor_primes)
-    beam_distances = calculate_distances(vectors, beams)
-    distances = beam_distances
-    remaining_capacity = queue_length * config["parallel_visit_count"]
-    batch_size = config["batch_size"]
-    search = closest_vectors_stepwise if stale_distances else closest_vectors
 
-    for _ in range(0, config["optimization_loops"]):
-        next_beams = torch.empty_like(beams)
-        next_beam_distances = torch.empty_like(beam_distances)
-        for start in range(0, num_vecs, batch_size):
-            end = min(start + batch_size, num_vecs)
-            exclude = excluding_self(start, end, queue_length, device)
-            queue = Queue(end - start, queue_length, queue_length + remaining_capacity, device=device)
-            seed_distances = beam_distances if stale_distances else distances
-            queue.insert(beams.narrow(0, start, end - start), seed_distances.narrow(0, start, end - start))
-            search(vectors[start:end], queue, vectors, beams, config, exclude)
-            next_beams.narrow(0, start, end - start).copy_(queue.indices.narrow(1, 0, queue_length))
-            next_beam_distances.narrow(0, start, end - start).copy_(queue.distances.narrow(1, 0, queue_length))
+    def __init__(self, vectors: Tensor, config: Dict, stale_distances: bool = False):
+        self.vectors = vectors
+        self.config = config
+        self.stale = stale_distances
+        (self.num_vecs, _) = vectors.size()
+        device = vectors.device
+        self.beam_size = config["beam_size"]
+        self.queue_length = self.beam_size * config["beam_queue_factor"]
+        neighbor_primes = primes(self.queue_length, device)
+        self.beams = generate_circulant_beams(self.num_vecs, neighbor_primes)
+        self.beam_distances = calculate_distances(vectors, self.beams)  # of the circulant graph
+        self.distances = self.beam_distances
+        self.stats: list = []  # one dict per finished optimisation loop
+        self.finished = False
 
-        if config["prune"]:
-            (beams, distances) = prune_(next_beams, next_beam_distances)
+    def batches_per_loop(self) -> int:
+        bs = self.config["batch_size"]
+        return (self.num_vecs + bs - 1) // bs
+
+    def steps(self):
+        """Generator: runs the build, yielding (loop, start, end, iterations) after each batch."""
+        config, vectors, device = self.config, self.vectors, self.vectors.device
+        ql = self.queue_length
+        remaining_capacity = ql * config["parallel_visit_count"]
+        batch_size = config["batch_size"]
+        search = closest_vectors_stepwise if self.stale else closest_vectors
+        for loop in range(0, config["optimization_loops"]):
+            loop_start = time.time()
+            iterations = 0
+            next_beams = torch.empty_like(self.beams)
+            next_beam_distances = torch.empty_like(self.beam_distances)
+            for start in range(0, self.num_vecs, batch_size):
+                end = min(start + batch_size, self.num_vecs)
+                exclude = excluding_self(start, end, ql, device)
+                queue = Queue(end - start, ql, ql + remaining_capacity, device=device)
+                seed_distances = self.beam_distances if self.stale else self.distances
+                queue.insert(self.beams.narrow(0, start, end - start), seed_distances.narrow(0, start, end - start))
+                t = search(vectors[start:end], queue, vectors, self.beams, config, exclude)
+                iterations += t
+                next_beams.narrow(0, start, end - start).copy_(queue.indices.narrow(1, 0, ql))
+                next_beam_distances.narrow(0, start, end - start).copy_(queue.distances.narrow(1, 0, ql))
+                last = end == self.num_vecs
+                if last:
+                    recall = self._finish_loop(next_beams, next_beam_distances)
+                    torch.cuda.synchronize(device)
+                    self.stats.append(dict(loop=loop, seconds=time.time() - loop_start, iterations=iterations,
+                                           self_recall=recall))
+                yield (loop, start, end, t)
+            if recall == 1.0:  # ann.py:187
+                break
+        self.finished = True
+
+    def _finish_loop(self, next_beams: Tensor, next_beam_distances: Tensor) -> float:
+        if self.config["prune"]:  # ann.py:171-177
+            (self.beams, self.distances) = prune_(next_beams, next_beam_distances)
         else:
-            (beams, distances) = (next_beams, next_beam_distances)
+            (self.beams, self.distances) = (next_beams, next_beam_distances)
+        prefix = min(self.num_vecs, 1000)  # ann.py:179-185
+        (_, recall) = ann_calculate_recall(self.vectors, self.beams.narrow_copy(1, 0, self.beam_size), self.config,
+                                           sample=self.vectors[:prefix])
+        return recall
 
-        prefix = min(num_vecs, 1000)
-        (_, recall) = ann_calculate_recall(vectors, beams.narrow_copy(1, 0, beam_size), config,
-                                           sample=vectors[:prefix])
-        if recall == 1.0:
-            break
-    out_distances = beam_distances if stale_distances else distances
-    return (beams.narrow_copy(1, 0, beam_size), out_distances.narrow_copy(1, 0, beam_size))
+    def result(self) -> Tuple[Tensor, Tensor]:
+        out_distances = self.beam_distances if self.stale else self.distances  # ann.py:190-193
+        return (self.beams.narrow_copy(1, 0, self.beam_size), out_distances.narrow_copy(1, 0, self.beam_size))
+
+
+def generate_ann(vectors: Tensor, config: Dict, stale_distances: bool = False,
+                 stats: Optional[list] = None) -> Tuple[Tensor, Tensor]:
+    """reference ann.py:109-193 (see GraphBuild).  stats, when given, receives
+    one dict per optimisation loop (wall seconds, beam-search iterations summed
+    over batches, self-recall)."""
+    build = GraphBuild(vectors, config, stale_distances)
+    for _ in build.steps():
+        pass
+    if stats is not None:
+        stats.extend(build.stats)
+    return build.result()
 
 
 def initial_queue(vectors: Tensor, config: Dict) -> Queue:
@@ -257,7 +302,8 @@ class ANN:
             else:
                 self.distances = distances.to(self.vectors.device).contiguous()
         else:
-            (self.beams, self.distances) = generate_ann(self.vectors, self.configuration)
+            self.build_stats: list = []
+            (self.beams, self.distances) = generate_ann(self.vectors, self.configuration, stats=self.build_stats)
         torch.cuda.synchronize(self.vectors.device)
         wall_end = time.time()
         self.log = self.configuration.copy()
