@@ -176,7 +176,8 @@ def main():
         "config": {"workload": args.workload, "n": n, "dim": dim, "degree": cfg["beam_size"],
                    "build_queue": cfg["beam_size"] * cfg["beam_queue_factor"], "batch_size": cfg["batch_size"],
                    "optimization_loops": cfg["optimization_loops"], "parallel_visit_count": 4,
-                   "seeding": "circulant (reference)", "queries": int(queries.shape[0])},
+                   "build_seeding": "circulant (reference)", "search_seeding": "dense, 32768 entry points",
+                   "queries": int(queries.shape[0])},
         "partial": not complete, "build_seconds": t_build, "loops": build.stats,
         "roofline": roofline,
     }
@@ -190,26 +191,33 @@ def main():
         torch.cuda.synchronize()
         t_knn = time.time() - t0
         flops = 2.0 * qdev.shape[0] * n * dim
-        sweep = []
-        chosen = None
-        for qs in (32, 64, 96, 128, 192, 256):
-            ann.search(qdev[:256].contiguous(), queue_size=qs)  # warm the workspace for this shape
-            torch.cuda.synchronize()
-            t0 = time.time()
-            res = ann.search(qdev, queue_size=qs)
-            torch.cuda.synchronize()
-            dt = time.time() - t0
-            found = res.indices[:, :10]
-            hits = (found.unsqueeze(2) == truth.unsqueeze(1)).any(dim=2).sum().item()
-            rec = hits / truth.numel()
-            sweep.append(dict(queue=qs, qps=qdev.shape[0] / dt, recall_at_10=rec))
-            if chosen is None and rec >= 0.95:
-                chosen = sweep[-1]
-        result["search"] = dict(sweep=sweep, at_recall_0_95=chosen, reached_0_95=chosen is not None,
-                                qps=(chosen or sweep[-1])["qps"], recall_at_10=(chosen or sweep[-1])["recall_at_10"])
+        def sweep_search(seeding):
+            sweep, chosen = [], None
+            for qs in (16, 32, 64, 96, 128, 192, 256):
+                ann.search(qdev[:256].contiguous(), queue_size=qs, seeding=seeding)  # warm this shape
+                torch.cuda.synchronize()
+                t0 = time.time()
+                res = ann.search(qdev, queue_size=qs, seeding=seeding)
+                torch.cuda.synchronize()
+                dt = time.time() - t0
+                found = res.indices[:, :10]
+                hits = (found.unsqueeze(2) == truth.unsqueeze(1)).any(dim=2).sum().item()
+                rec = hits / truth.numel()
+                sweep.append(dict(queue=qs, qps=qdev.shape[0] / dt, recall_at_10=rec))
+                if chosen is None and rec >= 0.95:
+                    chosen = sweep[-1]
+            best = chosen or max(sweep, key=lambda r: r["recall_at_10"])
+            return dict(seeding=seeding, sweep=sweep, reached_0_95=chosen is not None, queue=best["queue"],
+                        qps=best["qps"], recall_at_10=best["recall_at_10"])
+
+        # query-dependent seeds from dense MFMA tiles over 32,768 entry points (what reaches the recall target)
+        result["search"] = sweep_search("dense")
+        # the reference's query-independent circulant seeds, for comparison
+        result["search_reference_seeding"] = sweep_search("circulant")
+        log(f"[bench] search (dense seeds): {result['search']}")
+        log(f"[bench] search (circulant seeds): {result['search_reference_seeding']}")
         result["exact_knn"] = dict(seconds=t_knn, tflops=flops / t_knn / 1e12, peak_tflops=157.3,
                                    frac=flops / t_knn / 1e12 / 157.3, bound="mfma")
-        log(f"[bench] search sweep: {sweep}")
 
     if not args.no_cpu:
         # CPU leg: the oracle on the first rows of the same workload, first-loop state

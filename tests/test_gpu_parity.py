@@ -395,3 +395,42 @@ def test_knn_exact(n, dim, nq, k):
         assert abs(d_true - wd[r, c]) < 2e-6
     for r in range(nq):
         assert len(set(gi[r].tolist())) == k
+
+
+# ---------------------------------------------------------------- dense seeding (addition)
+def test_dense_seeded_search():
+    say("dense seeded search")
+    from vectorlink_gpu import ANN
+    from vectorlink_gpu.ann import entry_point_ids
+
+    rng = np.random.default_rng(21)
+    n, dim, nq = 3000, 32, 90
+    centres = unit(rng, 30, dim)
+    v = centres[rng.integers(0, 30, n)] + 0.05 * rng.standard_normal((n, dim)).astype(np.float32)
+    v = (v / np.linalg.norm(v, axis=1, keepdims=True)).astype(np.float32)
+    q = centres[rng.integers(0, 30, nq)] + 0.05 * rng.standard_normal((nq, dim)).astype(np.float32)
+    q = (q / np.linalg.norm(q, axis=1, keepdims=True)).astype(np.float32)
+    kw = dict(beam_size=12, beam_queue_factor=2, recall_search_queue_factor=2, batch_size=1000, optimization_loops=2)
+    c = cfg(**kw)
+    ann = ANN(dev(v), seeding="dense", entry_points=500, **kw)
+    eids = host(entry_point_ids(n, 500))
+    assert np.array_equal(eids, (np.arange(500, dtype=np.int64) * n) // 500)
+    res = ann.search(dev(q))
+    L = res.length
+    gi = host(res.indices)
+    # the seeds the GPU picked = the 16 nearest entry points (exact, up to float32 near-ties)
+    wi, wd = orc.knn_exact(q, v[eids], 16)
+    seeds_want = eids[wi]
+    # replay on the oracle from the oracle's seeds: identical answer unless a near-tie changed the seed set
+    oq = orc.Queue(nq, L, res.indices.shape[1])
+    oq.insert(seeds_want.astype(np.int32), orc.gather_distances(q, v, seeds_want.astype(np.int32)))
+    orc.closest_vectors(q, oq, v, host(ann.beams), c, None)
+    same = (gi[:, :L] == oq.indices[:, :L]).all(axis=1)
+    assert same.mean() > 0.97
+    assert np.array_equal(bits(host(res.distances)[same, :L]), bits(oq.distances[same, :L]))
+    # and it finds the true neighbours where circulant seeding cannot
+    t10, _ = orc.knn_exact(q, v, 10)
+    rec_dense = np.mean([len(set(a) & set(b)) / 10 for a, b in zip(gi[:, :10].tolist(), t10.tolist())])
+    rec_circ = ann.recall_at_k(dev(q), 10, seeding="circulant")
+    assert rec_dense > 0.9 and rec_dense == pytest.approx(ann.recall_at_k(dev(q), 10), abs=0.02)
+    assert rec_dense >= rec_circ

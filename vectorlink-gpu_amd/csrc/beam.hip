@@ -16,6 +16,7 @@
 // for progress (ann.py:68,90-91).
 #include "beam_ctrl.h"
 #include "rowsort.h"
+#include <stdlib.h>
 
 int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors, int64_t n_vectors,
                      int64_t dim, const int32_t *ids, const int32_t *visit, int64_t n_visit,
@@ -51,7 +52,7 @@ struct MergeArgs {
     int excl_cols;
     int32_t *v_ids;
     float *v_d;
-    int VL, Vt, Pv;
+    int VL, Vt, Pv, Pc;
     int32_t *seen;
     int32_t *seen_count;
     int E;
@@ -246,6 +247,223 @@ __global__ __launch_bounds__(kQueueThreads) void beam_merge_kernel(MergeArgs a) 
                  nullptr);
 }
 
+// ---- merge, second form ------------------------------------------------------
+// Same result as beam_merge_kernel on [0, length) of the search queue and on the
+// visit queue, for queues in the state Queue.insert leaves them (ordered by
+// (distance, id), distinct ids) and ids that always carry the same distance -
+// both hold for everything closest_vectors is handed by this package.  Instead
+// of two full-row sorts, the candidates are sorted once; what is already queued
+// (or excluded, or visited) is filtered out with binary searches; the few
+// survivors are merged into each sorted queue by rank.
+__device__ inline int key_lower_bound(const uint64_t *a, int n, uint64_t k) {
+    int lo = 0, hi = n;
+    while (lo < hi) {
+        int mid = (lo + hi) >> 1;
+        if (a[mid] < k) lo = mid + 1;
+        else hi = mid;
+    }
+    return lo;
+}
+
+// Order-preserving compaction of src[0:n) by predicate into dst; returns the
+// kept count (uniform).  wave_cnt: kQueueWaves ints of LDS.
+template <class Pred>
+__device__ inline int block_compact(const uint64_t *src, int n, uint64_t *dst, Pred keep, int *wave_cnt) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    int run = 0;
+    for (int base = 0; base < n; base += blockDim.x) {
+        int i = base + threadIdx.x;
+        bool k = i < n && keep(i);
+        uint64_t b = __ballot(k);
+        if (lane == 0) wave_cnt[wave] = __popcll(b);
+        __syncthreads();
+        if (k) {
+            int dest = run + __popcll(b & ((1ull << lane) - 1));
+            for (int w = 0; w < wave; ++w) dest += wave_cnt[w];
+            dst[dest] = src[i];
+        }
+        for (int w = 0; w < kQueueWaves; ++w) run += wave_cnt[w];
+        __syncthreads();
+    }
+    return run;
+}
+
+__global__ __launch_bounds__(kQueueThreads) void beam_merge2_kernel(MergeArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int Pc = a.Pc;
+    uint64_t *ck = reinterpret_cast<uint64_t *>(smem);  // candidates, sorted
+    uint64_t *cc = ck + Pc;                             // filtered candidates
+    uint64_t *qa = cc + Pc;                             // search queue [0, L)
+    uint64_t *va = qa + a.L;                            // visit queue [Vt, VL)
+    int32_t *seen_a = reinterpret_cast<int32_t *>(va + a.VL);
+    int32_t *seen_b = seen_a + a.E;
+    int32_t *exl = seen_b + a.E;
+    __shared__ int wave_cnt[kQueueWaves];
+    __shared__ int n_ex_s;
+    __shared__ int32_t newv[kMaxVisit];
+    __shared__ int n_new_s;
+
+    BeamCtrl *c = a.ctrl;
+    if (c->stop) return;
+    const int t = a.iter;
+    const int64_t row = blockIdx.x;
+    const int lane = threadIdx.x & (kWave - 1);
+    int cnt = a.seen_count[row];
+    int *first_next = &c->first[(t + 1) & 1];
+    if (t >= 2 && c->first[(t - 1) & 1] >= a.E) {
+        if (threadIdx.x == 0) atomicMax(first_next, cnt);
+        return;
+    }
+    const int first = c->first[t & 1];
+    const bool seen_full = first >= a.E;
+    const bool checking = (t % a.readahead) == 0;
+
+    int32_t *qi = a.q_ids + row * a.cap;
+    float *qd = a.q_d + row * a.cap;
+    int32_t *vi = a.v_ids + row * a.VL;
+    float *vd = a.v_d + row * a.VL;
+    const int32_t *ci = a.cand_ids + row * a.m;
+    const float *cd = a.cand_d + row * a.m;
+    const int nva = a.VL - a.Vt;
+
+    // ---- load -----------------------------------------------------------------
+    if (threadIdx.x == 0) {
+        n_ex_s = a.excl ? a.excl_cols : 0;
+        n_new_s = 0;
+    }
+    __syncthreads();
+    if (a.excl) {
+        const int32_t *ex = a.excl + row * a.excl_cols;
+        for (int i = threadIdx.x; i < a.excl_cols; i += blockDim.x) {
+            int32_t e = ex[i];
+            exl[i] = e;
+            if (e == VL_MAXINT) atomicMin(&n_ex_s, i);
+        }
+    }
+    for (int i = threadIdx.x; i < Pc; i += blockDim.x) ck[i] = i < a.m ? vl_make_key(ci[i], cd[i]) : kPadKey;
+    for (int i = threadIdx.x; i < a.L; i += blockDim.x) qa[i] = vl_make_key(qi[i], qd[i]);
+    for (int i = threadIdx.x; i < nva; i += blockDim.x) va[i] = vl_make_key(vi[a.Vt + i], vd[a.Vt + i]);
+    // the ids popped at the start of this iteration (queue.py:87-95), before the row is rewritten
+    int32_t popped = VL_MAXINT;
+    if (threadIdx.x < kWave && threadIdx.x < a.Vt) popped = vi[threadIdx.x];
+    if (!seen_full) {
+        const int32_t *srow = a.seen + row * a.E;
+        for (int i = threadIdx.x; i < cnt; i += blockDim.x) seen_a[i] = srow[i];
+    }
+    block_bitonic_sort(ck, Pc);
+    const int n_ex = n_ex_s;
+    // real candidates sort before every empty pair and pad
+    const int n_real = key_lower_bound(ck, Pc, vl_make_key(VL_MAXINT, VL_MAXFLOAT));
+
+    // ---- search_queue.insert : ann.py:75-80 -------------------------------------
+    auto keep_search = [&](int i) -> bool {
+        uint64_t k = ck[i];
+        int32_t id = vl_key_id(k);
+        if (i > 0 && id == vl_key_id(ck[i - 1])) return false;   // neighbouring duplicate (kernels.py:314-349)
+        for (int e = 0; e < n_ex; ++e)
+            if (exl[e] == id) return false;                      // queue.py:52-53
+        int p = key_lower_bound(qa, a.L, k);
+        return !(p < a.L && qa[p] == k);                         // already queued
+    };
+    const int n_s = block_compact(ck, n_real, cc, keep_search, wave_cnt);
+    bool diff = false;
+    for (int i = threadIdx.x; i < a.L; i += blockDim.x) {
+        uint64_t k = qa[i];
+        int r = i + key_lower_bound(cc, n_s, k);
+        if (r < a.L) {
+            qi[r] = vl_key_id(k);
+            qd[r] = vl_key_dist(k);
+        }
+    }
+    for (int j = threadIdx.x; j < n_s; j += blockDim.x) {
+        uint64_t k = cc[j];
+        int r = j + key_lower_bound(qa, a.L, k);
+        if (r < a.L) {
+            qi[r] = vl_key_id(k);
+            qd[r] = vl_key_dist(k);
+            diff = true;  // a new id inside the first L slots: the row changed (queue.py:57-59)
+        }
+    }
+    if (checking && __ballot(diff) && lane == 0) atomicOr(&c->changed[(t / a.readahead) & 63], 1);
+
+    if (seen_full) {
+        if (threadIdx.x == 0) atomicMax(first_next, cnt);
+        return;
+    }
+    __syncthreads();  // cc is reused below
+
+    // ---- add_new_to_seen_ : utils.py:61-82 ---------------------------------------
+    const int n_add = min(a.E - first, a.Vt);
+    if (threadIdx.x < kWave) {
+        const int j = threadIdx.x;
+        int32_t x = j < n_add ? popped : VL_MAXINT;
+        bool valid = j < n_add && x != VL_MAXINT && !sorted_contains(seen_a, cnt, x);
+        int rank = 0;
+        for (int i = 0; i < n_add; ++i) {
+            int32_t y = __shfl(popped, i);
+            if (i < j && y == x) valid = false;
+        }
+        uint64_t vm = __ballot(valid);
+        for (int i = 0; i < n_add; ++i) {
+            int32_t y = __shfl(popped, i);
+            if (((vm >> i) & 1) && y < x) ++rank;
+        }
+        if (valid) newv[rank] = x;
+        if (j == 0) n_new_s = __popcll(vm);
+    }
+    __syncthreads();
+    const int n_new = n_new_s;
+    for (int p = threadIdx.x; p < cnt; p += blockDim.x) {
+        int32_t v = seen_a[p];
+        int shift = 0;
+        for (int i = 0; i < n_new; ++i) shift += newv[i] < v;
+        seen_b[p + shift] = v;
+    }
+    if (threadIdx.x < n_new) seen_b[lower_bound(seen_a, cnt, newv[threadIdx.x]) + threadIdx.x] = newv[threadIdx.x];
+    __syncthreads();
+    cnt += n_new;
+    if (n_new) {
+        int32_t *srow = a.seen + row * a.E;
+        for (int i = threadIdx.x; i < cnt; i += blockDim.x) srow[i] = seen_b[i];
+    }
+    if (threadIdx.x == 0) {
+        a.seen_count[row] = cnt;
+        atomicMax(first_next, cnt);
+    }
+
+    // ---- visit_queue.insert(candidates, exclude=seen) : ann.py:85-88 --------------
+    auto keep_visit = [&](int i) -> bool {
+        uint64_t k = ck[i];
+        int32_t id = vl_key_id(k);
+        if (i > 0 && id == vl_key_id(ck[i - 1])) return false;
+        if (sorted_contains(seen_b, cnt, id)) return false;      // kernels.py:471-488
+        int p = key_lower_bound(va, nva, k);
+        return !(p < nva && va[p] == k);
+    };
+    const int n_v = block_compact(ck, n_real, cc, keep_visit, wave_cnt);
+    for (int i = threadIdx.x; i < nva; i += blockDim.x) {
+        uint64_t k = va[i];
+        int r = i + key_lower_bound(cc, n_v, k);
+        if (r < a.VL) {
+            vi[r] = vl_key_id(k);
+            vd[r] = vl_key_dist(k);
+        }
+    }
+    for (int j = threadIdx.x; j < n_v; j += blockDim.x) {
+        uint64_t k = cc[j];
+        int r = j + key_lower_bound(va, nva, k);
+        if (r < a.VL) {
+            vi[r] = vl_key_id(k);
+            vd[r] = vl_key_dist(k);
+        }
+    }
+    for (int r = nva + n_v + threadIdx.x; r < a.VL; r += blockDim.x) {  // the popped slots end up here, empty
+        vi[r] = VL_MAXINT;
+        vd[r] = VL_MAXFLOAT;
+    }
+}
+
 struct BeamLayout {
     int64_t m, VL, Vt, E, head;
     int64_t off_cand_ids, off_cand_d, off_v_ids, off_v_d, off_seen, off_seen_count, off_ctrl, total;
@@ -337,8 +555,17 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
     a.excl = p->excl_cols > 0 ? exclude : nullptr; a.excl_cols = a.excl ? (int)p->excl_cols : 0;
     a.v_ids = v_ids; a.v_d = v_d; a.VL = (int)l.VL; a.Vt = (int)l.Vt; a.Pv = vl_next_pow2(l.VL + l.m);
     a.seen = seen; a.seen_count = seen_count; a.E = (int)l.E;
+    a.Pc = vl_next_pow2(l.m);
+    if (a.Pc < 2) a.Pc = 2;
+    // VL_BEAM_MERGE=sort selects the full-row-sort form of the merge step (exact for queue rows in any state)
+    static const bool use_sort_merge = [] {
+        const char *e = getenv("VL_BEAM_MERGE");
+        return e && e[0] == 's';
+    }();
     const int Pmax = a.Ps > a.Pv ? a.Ps : a.Pv;
-    const size_t smem = (size_t)Pmax * 8 + (size_t)a.L * 4 + (size_t)a.E * 8 + (size_t)a.excl_cols * 4;
+    const size_t smem = use_sort_merge
+        ? (size_t)Pmax * 8 + (size_t)a.L * 4 + (size_t)a.E * 8 + (size_t)a.excl_cols * 4
+        : (size_t)a.Pc * 16 + (size_t)(a.L + a.VL) * 8 + (size_t)a.E * 8 + (size_t)a.excl_cols * 4;
     VL_REQUIRE(smem <= 60 * 1024, "queues of this size need %zu bytes of LDS (limit 61440)", smem);
 
     const int R = (int)p->speculative_readahead;
@@ -359,8 +586,11 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
             if (rc < 0) return rc;
             if (prof) VL_HIP(hipEventRecord(ev[3 * r + 1], st));
             a.iter = (int)t;
-            hipLaunchKernelGGL(beam_merge_kernel, dim3((unsigned)p->n_rows), dim3(kQueueThreads), smem, st, a);
-            VL_LAUNCH_CHECK("beam_merge_kernel");
+            if (use_sort_merge)
+                hipLaunchKernelGGL(beam_merge_kernel, dim3((unsigned)p->n_rows), dim3(kQueueThreads), smem, st, a);
+            else
+                hipLaunchKernelGGL(beam_merge2_kernel, dim3((unsigned)p->n_rows), dim3(kQueueThreads), smem, st, a);
+            VL_LAUNCH_CHECK("beam merge kernel");
             if (prof) VL_HIP(hipEventRecord(ev[3 * r + 2], st));
         }
         int changed = 0;

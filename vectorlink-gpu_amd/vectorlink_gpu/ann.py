@@ -241,6 +241,36 @@ def initial_search_queue(vectors: Tensor, query_vectors: Tensor, config: Dict,
     return queue
 
 
+DENSE_SEEDS = 16  # seeds per query taken from the entry-point tiles (the exact-kNN kernel keeps 16 per lane)
+
+
+def entry_point_ids(vector_count: int, entry_points: int, device=DEVICE) -> Tensor:
+    """Ids of the entry-point sample: entry_points ids spread evenly over [0, vector_count)."""
+    s = min(entry_points, vector_count)
+    return ((torch.arange(s, dtype=torch.int64, device=device) * vector_count) // s).to(torch.int32)
+
+
+def dense_search_queue(vectors: Tensor, query_vectors: Tensor, config: Dict, entry_ids: Tensor,
+                       entry_vectors: Tensor, queue_size: Optional[int] = None) -> Queue:
+    """Query-dependent seeding (not in the reference, whose seeds (b + p_k) % N ignore
+    the query, utils.py:26-32): the seeds of a query are its DENSE_SEEDS nearest
+    entry points, found with one dense query x entry-point pass on fp32 MFMA tiles.
+    Their distances are then re-evaluated with the gathered-distance kernel so that
+    a seed met again during the search carries identical bits.  Same queue shape as
+    initial_search_queue (ann.py:217-232); slots beyond the seeds start empty."""
+    if queue_size is None:
+        queue_size = config["recall_search_queue_factor"] * config["beam_size"]
+    (batch_size, _) = query_vectors.size()
+    extra_capacity = max(queue_size, config["parallel_visit_count"] * config["beam_size"])
+    queue = Queue(batch_size, queue_size, queue_size + extra_capacity, device=vectors.device)
+    k = min(DENSE_SEEDS, entry_ids.size(0), queue_size)
+    (local, _) = knn_exact(query_vectors, entry_vectors, k)
+    seeds = entry_ids[local.long()].contiguous()
+    d = query_cosine_distances(query_vectors, vectors, seeds)
+    queue.insert(seeds, d)
+    return queue
+
+
 def ann_calculate_recall(vectors: Tensor, beams: Tensor, config: Dict, sample: Optional[Tensor] = None,
                          verbose: bool = False):
     """reference ann.py:235-259: share of sample rows whose best hit is themselves"""
@@ -276,8 +306,17 @@ class ANN:
         speculative_readahead: int = 5,
         beams: Optional[Tensor] = None,
         distances: Optional[Tensor] = None,
+        seeding: str = "circulant",
+        entry_points: int = 32_768,
     ):
+        """seeding / entry_points are additions: "circulant" seeds searches as the
+        reference does; "dense" seeds them from the nearest of `entry_points`
+        evenly spread vectors (see dense_search_queue)."""
         assert vectors.dim() == 2 and vectors.dtype == torch.float32
+        assert seeding in ("circulant", "dense")
+        self.seeding = seeding
+        self.entry_points = entry_points
+        self._entry = None
         (count, dim) = vectors.size()
         self.configuration: Dict = {
             "prune": prune,
@@ -322,26 +361,41 @@ class ANN:
         """reference ann.py:466-467 (a stub there as well)"""
         return None
 
-    def search(self, query: Tensor, queue_size: Optional[int] = None) -> Queue:
+    def _entry_tables(self):
+        if self._entry is None:
+            ids = entry_point_ids(self.vectors.size(0), self.entry_points, self.vectors.device)
+            self._entry = (ids, self.vectors[ids.long()].contiguous())
+        return self._entry
+
+    def search(self, query: Tensor, queue_size: Optional[int] = None, seeding: Optional[str] = None) -> Queue:
         """reference ann.py:469-477: takes a batch of query vectors, returns the
         search Queue; the answer is queue.indices[:, :k] / queue.distances[:, :k].
-        queue_size overrides the configured search-queue length."""
+        queue_size overrides the configured search-queue length, seeding the
+        instance's seeding mode."""
         assert query.dim() == 2 and query.dtype == torch.float32
         if not query.is_cuda:
             query = query.to(self.vectors.device)
         query = query.contiguous()
-        search_queue = initial_search_queue(self.vectors, query, self.configuration, queue_size)
+        seeding = seeding or self.seeding
+        assert seeding in ("circulant", "dense")
+        if seeding == "dense":
+            (entry_ids, entry_vectors) = self._entry_tables()
+            search_queue = dense_search_queue(self.vectors, query, self.configuration, entry_ids, entry_vectors,
+                                              queue_size)
+        else:
+            search_queue = initial_search_queue(self.vectors, query, self.configuration, queue_size)
         closest_vectors(query, search_queue, self.vectors, self.beams, self.configuration, None)
         return search_queue
 
-    def recall_at_k(self, query: Tensor, k: int = 10, queue_size: Optional[int] = None) -> float:
+    def recall_at_k(self, query: Tensor, k: int = 10, queue_size: Optional[int] = None,
+                    seeding: Optional[str] = None) -> float:
         """Share of the exact k nearest neighbours (brute force on MFMA tiles)
         that search() returns in its first k slots.  Not in the reference,
         whose recall() is self-recall@1."""
         if not query.is_cuda:
             query = query.to(self.vectors.device)
         query = query.contiguous()
-        found = self.search(query, queue_size).indices[:, :k]
+        found = self.search(query, queue_size, seeding).indices[:, :k]
         (truth, _) = knn_exact(query, self.vectors, k)
         hits = (found.unsqueeze(2) == truth.unsqueeze(1)).any(dim=2).sum().item()
         return hits / truth.numel()
