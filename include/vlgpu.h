@@ -167,10 +167,11 @@ int64_t vl_closest_vectors(const vl_beam_params *p,
 
 /* Per-kernel timing of vl_closest_vectors (no counterpart in the reference,
  * whose log.py:7-17 times whole calls): with enable != 0 every expand / merge
- * launch is bracketed by HIP events on the caller's stream.  out (7 doubles,
+ * launch is bracketed by HIP events on the caller's stream.  out (8 doubles,
  * may be NULL) receives the sums since the last reset: expand ms, merge ms,
  * expand launches, merge launches, candidate rows fetched, query rows,
- * iterations.  Not thread safe. */
+ * iterations, candidate distances asked for (fetched + served by the per-row
+ * cache of already evaluated pairs).  Not thread safe. */
 int vl_beam_profile(int enable, int reset, double *out);
 
 /* ---- pruning (kernels.py:441-468 prune_) ------------------------------ */

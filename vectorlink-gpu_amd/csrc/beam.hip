@@ -22,7 +22,8 @@ int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors,
                      int64_t dim, const int32_t *ids, const int32_t *visit, int64_t n_visit,
                      const int32_t *beams, int64_t n_nodes, int64_t width, int64_t m,
                      int32_t *idx_out, float *dist_out, BeamCtrl *ctrl, int iter, int readahead,
-                     int seen_cols, int64_t visit_stride, int count_evals, hipStream_t st);
+                     int seen_cols, int64_t visit_stride, int count_evals, uint64_t *memo, int memo_slots,
+                     hipStream_t st);
 
 namespace {
 
@@ -33,7 +34,7 @@ constexpr int kMaxVisit = 64;  // parallel_visit_count handled by one wavefront
 struct BeamProfile {
     int enabled = 0;
     double expand_ms = 0, merge_ms = 0;
-    int64_t expand_launches = 0, merge_launches = 0, evals = 0, rows = 0, iterations = 0;
+    int64_t expand_launches = 0, merge_launches = 0, evals = 0, rows = 0, iterations = 0, wanted = 0;
 };
 BeamProfile g_prof;
 
@@ -77,6 +78,12 @@ __device__ inline int lower_bound(const int32_t *a, int n, int32_t v) {
     return lo;
 }
 
+__global__ void beam_memo_clear_kernel(uint64_t *memo, int64_t n) {
+    // an empty slot holds id VL_MAXINT, which no probe asks for
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        memo[i] = (uint64_t)(uint32_t)VL_MAXINT;
+}
+
 __global__ __launch_bounds__(kQueueThreads) void beam_init_kernel(BeamCtrl *ctrl, int64_t n_rows, const int32_t *q_ids,
                                                                  const float *q_d, int cap, int head, int32_t *v_ids,
                                                                  float *v_d, int VL, int32_t *seen_count) {
@@ -89,6 +96,7 @@ __global__ __launch_bounds__(kQueueThreads) void beam_init_kernel(BeamCtrl *ctrl
     if (t < 64) {
         ctrl->changed[t] = 0;
         ctrl->evals[t] = 0;
+        ctrl->wanted[t] = 0;
     }
     if (t < n_rows) seen_count[t] = 0;
     if (t < n_rows * VL) {  // Queue.initialize_from_queue, queue.py:30-35
@@ -283,13 +291,14 @@ __device__ inline int block_compact(const uint64_t *src, int n, uint64_t *dst, P
             for (int w = 0; w < wave; ++w) dest += wave_cnt[w];
             dst[dest] = src[i];
         }
-        for (int w = 0; w < kQueueWaves; ++w) run += wave_cnt[w];
+        for (int w = 0; w < (int)(blockDim.x / kWave); ++w) run += wave_cnt[w];
         __syncthreads();
     }
     return run;
 }
 
-__global__ __launch_bounds__(kQueueThreads) void beam_merge2_kernel(MergeArgs a) {
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void beam_merge2_kernel(MergeArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int Pc = a.Pc;
     uint64_t *ck = reinterpret_cast<uint64_t *>(smem);  // candidates, sorted
@@ -385,7 +394,10 @@ __global__ __launch_bounds__(kQueueThreads) void beam_merge2_kernel(MergeArgs a)
             diff = true;  // a new id inside the first L slots: the row changed (queue.py:57-59)
         }
     }
-    if (checking && __ballot(diff) && lane == 0) atomicOr(&c->changed[(t / a.readahead) & 63], 1);
+    if (checking && __ballot(diff) && lane == 0) {
+        int *flag = &c->changed[(t / a.readahead) & 63];
+        if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) atomicOr(flag, 1);
+    }
 
     if (seen_full) {
         if (threadIdx.x == 0) atomicMax(first_next, cnt);
@@ -429,7 +441,8 @@ __global__ __launch_bounds__(kQueueThreads) void beam_merge2_kernel(MergeArgs a)
     }
     if (threadIdx.x == 0) {
         a.seen_count[row] = cnt;
-        atomicMax(first_next, cnt);
+        // the running maximum only grows: most rows find it already at their fill and skip the atomic
+        if (__hip_atomic_load(first_next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < cnt) atomicMax(first_next, cnt);
     }
 
     // ---- visit_queue.insert(candidates, exclude=seen) : ann.py:85-88 --------------
@@ -466,7 +479,8 @@ __global__ __launch_bounds__(kQueueThreads) void beam_merge2_kernel(MergeArgs a)
 
 struct BeamLayout {
     int64_t m, VL, Vt, E, head;
-    int64_t off_cand_ids, off_cand_d, off_v_ids, off_v_d, off_seen, off_seen_count, off_ctrl, total;
+    int64_t off_cand_ids, off_cand_d, off_v_ids, off_v_d, off_seen, off_seen_count, off_ctrl, off_memo, total;
+    int memo_slots;
 };
 
 inline int64_t align256(int64_t x) { return (x + 255) & ~255ll; }
@@ -499,6 +513,17 @@ int beam_layout(const vl_beam_params *p, BeamLayout *l) {
     l->off_seen = o; o = align256(o + p->n_rows * l->E * 4);
     l->off_seen_count = o; o = align256(o + p->n_rows * 4);
     l->off_ctrl = o; o = align256(o + (int64_t)sizeof(BeamCtrl));
+    // per-row cache of evaluated (id, distance) pairs: 32 slots per candidate of one iteration, 1Ki..16Ki
+    static const int memo_env = [] {
+        const char *e = getenv("VL_BEAM_MEMO");
+        return e ? atoi(e) : -1;
+    }();
+    int slots = vl_next_pow2(32 * l->m);
+    if (slots < 1024) slots = 1024;
+    if (slots > 16384) slots = 16384;
+    if (memo_env >= 0) slots = memo_env;
+    l->memo_slots = slots;
+    l->off_memo = o; o = align256(o + p->n_rows * (int64_t)slots * 8);
     l->total = o;
     return VL_OK;
 }
@@ -546,6 +571,11 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
                            (int)l.head, v_ids, v_d, (int)l.VL, seen_count);
         VL_LAUNCH_CHECK("beam_init_kernel");
     }
+    uint64_t *memo = (uint64_t *)(ws + l.off_memo);
+    if (l.memo_slots > 0) {
+        hipLaunchKernelGGL(beam_memo_clear_kernel, dim3(4096), dim3(256), 0, st, memo, p->n_rows * (int64_t)l.memo_slots);
+        VL_LAUNCH_CHECK("beam_memo_clear_kernel");
+    }
 
     MergeArgs a;
     a.ctrl = ctrl; a.readahead = (int)p->speculative_readahead; a.n_rows = p->n_rows;
@@ -561,6 +591,10 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
     static const bool use_sort_merge = [] {
         const char *e = getenv("VL_BEAM_MERGE");
         return e && e[0] == 's';
+    }();
+    static const int merge_threads = [] {
+        const char *e = getenv("VL_BEAM_MERGE_THREADS");
+        return e ? atoi(e) : 256;
     }();
     const int Pmax = a.Ps > a.Pv ? a.Ps : a.Pv;
     const size_t smem = use_sort_merge
@@ -582,14 +616,18 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
             if (prof) VL_HIP(hipEventRecord(ev[3 * r], st));
             rc = vl_launch_expand(queries, p->n_rows, vectors, p->n_vectors, p->dim, nullptr, v_ids, l.Vt, beams,
                                   p->n_vectors, p->width, l.m, cand_ids, cand_d, ctrl, (int)t, R, (int)l.E, l.VL,
-                                  prof ? 1 : 0, st);
+                                  prof ? 1 : 0, memo, l.memo_slots, st);
             if (rc < 0) return rc;
             if (prof) VL_HIP(hipEventRecord(ev[3 * r + 1], st));
             a.iter = (int)t;
             if (use_sort_merge)
                 hipLaunchKernelGGL(beam_merge_kernel, dim3((unsigned)p->n_rows), dim3(kQueueThreads), smem, st, a);
+            else if (merge_threads == 64)
+                hipLaunchKernelGGL(beam_merge2_kernel<64>, dim3((unsigned)p->n_rows), dim3(64), smem, st, a);
+            else if (merge_threads == 128)
+                hipLaunchKernelGGL(beam_merge2_kernel<128>, dim3((unsigned)p->n_rows), dim3(128), smem, st, a);
             else
-                hipLaunchKernelGGL(beam_merge2_kernel, dim3((unsigned)p->n_rows), dim3(kQueueThreads), smem, st, a);
+                hipLaunchKernelGGL(beam_merge2_kernel<256>, dim3((unsigned)p->n_rows), dim3(256), smem, st, a);
             VL_LAUNCH_CHECK("beam merge kernel");
             if (prof) VL_HIP(hipEventRecord(ev[3 * r + 2], st));
         }
@@ -615,6 +653,9 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
         VL_HIP(hipMemcpyAsync(ev_counts, ctrl->evals, sizeof(ev_counts), hipMemcpyDeviceToHost, st));
         VL_HIP(hipStreamSynchronize(st));
         for (int i = 0; i < 64; ++i) g_prof.evals += (int64_t)ev_counts[i];
+        VL_HIP(hipMemcpyAsync(ev_counts, ctrl->wanted, sizeof(ev_counts), hipMemcpyDeviceToHost, st));
+        VL_HIP(hipStreamSynchronize(st));
+        for (int i = 0; i < 64; ++i) g_prof.wanted += (int64_t)ev_counts[i];
         g_prof.rows += p->n_rows;
         g_prof.iterations += t;
         for (int i = 0; i < 3 * R; ++i) (void)hipEventDestroy(ev[i]);
@@ -624,14 +665,16 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
 
 // Profiling switch for vl_closest_vectors: when enabled every expand / merge
 // launch is bracketed by HIP events on the caller's stream and the fetched
-// candidate rows are counted.  out[0..6] = expand ms, merge ms, expand
+// candidate rows are counted.  out[0..7] = expand ms, merge ms, expand
 // launches, merge launches, candidate rows fetched, query rows, iterations,
+// candidate distances asked for (fetched + served by the per-row cache),
 // summed since the last reset.
 VL_EXPORT int vl_beam_profile(int enable, int reset, double *out) {
     if (out) {
         out[0] = g_prof.expand_ms; out[1] = g_prof.merge_ms;
         out[2] = (double)g_prof.expand_launches; out[3] = (double)g_prof.merge_launches;
         out[4] = (double)g_prof.evals; out[5] = (double)g_prof.rows; out[6] = (double)g_prof.iterations;
+        out[7] = (double)g_prof.wanted;
     }
     if (reset) g_prof = BeamProfile();
     g_prof.enabled = enable;

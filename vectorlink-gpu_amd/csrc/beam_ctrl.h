@@ -15,6 +15,7 @@ struct BeamCtrl {
     int first[2];
     int changed[64];
     unsigned long long evals[64];  // profiling only: candidate rows actually fetched, striped by workgroup
+    unsigned long long wanted[64]; // profiling only: candidate distances asked for (fetched or served by the cache)
 };
 
 // State of iteration t as seen by a kernel launched for it:

@@ -28,13 +28,21 @@ __device__ __forceinline__ float clamp_distance(float cos_theta) {
     return r;
 }
 
+// Per-row cache of distances already evaluated in this search: slot = hash(id),
+// entry = (distance bits << 32) | id, written and read as one 8-byte access.
+__device__ __forceinline__ uint32_t memo_hash(int32_t id, int shift) { return ((uint32_t)id * 2654435761u) >> shift; }
+__device__ __forceinline__ void memo_store(uint64_t *memo_row, int shift, int32_t id, float d) {
+    memo_row[memo_hash(id, shift)] = ((uint64_t)__builtin_bit_cast(uint32_t, d) << 32) | (uint32_t)id;
+}
+
 // One wavefront: lane j holds candidate id `my_id` (valid when `ok`); the
 // distance of candidate lane j to the query goes to out_d[j].
 template <int CPL, int LPR, int U>
 __device__ __forceinline__ void wave_distances(const float *__restrict__ q_row,
                                                const float *__restrict__ vectors, int dim,
                                                int nchunks, int32_t my_id, bool ok,
-                                               float *__restrict__ out_d) {
+                                               float *__restrict__ out_d, uint64_t *memo_row,
+                                               int memo_shift) {
     constexpr int G = kWave / LPR;
     const int lane = threadIdx.x & (kWave - 1);
     const int grp = lane / LPR;
@@ -66,6 +74,7 @@ __device__ __forceinline__ void wave_distances(const float *__restrict__ q_row,
 
         float4 r[U][CPL];
         int mysrc[U];
+        int32_t ids[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             int s = src[u][0];
@@ -78,6 +87,7 @@ __device__ __forceinline__ void wave_distances(const float *__restrict__ q_row,
             } else {
                 id = __shfl(my_id, s >= 0 ? s : 0);
             }
+            ids[u] = id;
             const float4 *row = reinterpret_cast<const float4 *>(vectors + (int64_t)id * dim);
 #pragma unroll
             for (int i = 0; i < CPL; ++i) {
@@ -97,7 +107,11 @@ __device__ __forceinline__ void wave_distances(const float *__restrict__ q_row,
             }
 #pragma unroll
             for (int h = LPR / 2; h >= 1; h >>= 1) acc = acc + __shfl_xor(acc, h);
-            if (lig == 0 && mysrc[u] >= 0) out_d[mysrc[u]] = clamp_distance(acc);
+            if (lig == 0 && mysrc[u] >= 0) {
+                float d = clamp_distance(acc);
+                out_d[mysrc[u]] = d;
+                if (memo_row) memo_store(memo_row, memo_shift, ids[u], d);
+            }
         }
     }
 }
@@ -106,7 +120,8 @@ __device__ __forceinline__ void wave_distances(const float *__restrict__ q_row,
 __device__ __forceinline__ void wave_distances_generic(const float *__restrict__ q_row,
                                                        const float *__restrict__ vectors, int dim,
                                                        int nchunks, int32_t my_id, bool ok,
-                                                       float *__restrict__ out_d) {
+                                                       float *__restrict__ out_d, uint64_t *memo_row,
+                                                       int memo_shift) {
     const int lane = threadIdx.x & (kWave - 1);
     uint64_t mask = __ballot(ok);
     while (mask) {
@@ -124,7 +139,11 @@ __device__ __forceinline__ void wave_distances_generic(const float *__restrict__
         }
 #pragma unroll
         for (int h = kWave / 2; h >= 1; h >>= 1) acc = acc + __shfl_xor(acc, h);
-        if (lane == 0) out_d[s] = clamp_distance(acc);
+        if (lane == 0) {
+            float d = clamp_distance(acc);
+            out_d[s] = d;
+            if (memo_row) memo_store(memo_row, memo_shift, id, d);
+        }
     }
 }
 
@@ -142,6 +161,8 @@ struct ExpandArgs {
     int seen_cols;         //   columns of the visited list
     int visit_stride;      // row stride of `visit` in elements
     int count_evals;       //   profiling: add the number of fetched rows to ctrl->evals
+    uint64_t *memo;        // optional per-row cache of (id, distance) pairs already evaluated (else null)
+    int memo_shift;        //   32 - log2(slots per row)
     int64_t n_rows;
     int64_t n_vectors;
     int64_t n_nodes;
@@ -196,11 +217,28 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs a) {
             id = a.ids[row * a.m + slot];
         }
     }
-    const bool ok = has && id != VL_MAXINT && id >= 0 && (int64_t)id < a.n_vectors;
+    bool ok = has && id != VL_MAXINT && id >= 0 && (int64_t)id < a.n_vectors;
     float *out_d = a.dist_out + row * a.m + c0;
     if (has) {
         if (a.idx_out) a.idx_out[row * a.m + slot] = ok ? id : VL_MAXINT;
         if (!ok) out_d[lane] = VL_MAXFLOAT;
+    }
+    if (a.count_evals) {
+        uint64_t wm = __ballot(ok);
+        if (lane == 0 && wm) atomicAdd(&a.ctrl->wanted[blockIdx.x & 63], (unsigned long long)__popcll(wm));
+    }
+    // A distance evaluated earlier in this search for the same (row, id) is
+    // reused: the cached bits are the ones this kernel would produce again.
+    uint64_t *memo_row = nullptr;
+    if (a.memo) {
+        memo_row = a.memo + ((uint64_t)row << (32 - a.memo_shift));
+        if (ok) {
+            uint64_t e = memo_row[memo_hash(id, a.memo_shift)];
+            if ((int32_t)(uint32_t)e == id) {
+                out_d[lane] = __builtin_bit_cast(float, (uint32_t)(e >> 32));
+                ok = false;
+            }
+        }
     }
     if (a.count_evals) {
         uint64_t okm = __ballot(ok);
@@ -208,9 +246,9 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs a) {
     }
     const float *q_row = a.queries + row * a.dim;
     if constexpr (GENERIC)
-        wave_distances_generic(q_row, a.vectors, a.dim, a.nchunks, id, ok, out_d);
+        wave_distances_generic(q_row, a.vectors, a.dim, a.nchunks, id, ok, out_d, memo_row, a.memo_shift);
     else
-        wave_distances<CPL, LPR, U>(q_row, a.vectors, a.dim, a.nchunks, id, ok, out_d);
+        wave_distances<CPL, LPR, U>(q_row, a.vectors, a.dim, a.nchunks, id, ok, out_d, memo_row, a.memo_shift);
 }
 
 template <int CPL, int LPR, int U>
@@ -225,7 +263,8 @@ int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors,
                      int64_t dim, const int32_t *ids, const int32_t *visit, int64_t n_visit,
                      const int32_t *beams, int64_t n_nodes, int64_t width, int64_t m,
                      int32_t *idx_out, float *dist_out, BeamCtrl *ctrl, int iter, int readahead,
-                     int seen_cols, int64_t visit_stride, int count_evals, hipStream_t st) {
+                     int seen_cols, int64_t visit_stride, int count_evals, uint64_t *memo, int memo_slots,
+                     hipStream_t st) {
     if (n_rows == 0 || m == 0) return VL_OK;
     VL_REQUIRE(dim >= 1 && dim <= (1 << 24), "dim %lld out of range", (long long)dim);
     VL_REQUIRE(m <= (1 << 24), "row of %lld candidates is too wide", (long long)m);
@@ -235,6 +274,14 @@ int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors,
     a.ctrl = ctrl; a.iter = iter; a.readahead = readahead; a.seen_cols = seen_cols;
     a.visit_stride = (int)visit_stride;
     a.count_evals = ctrl ? count_evals : 0;
+    a.memo = memo_slots > 0 ? memo : nullptr;
+    a.memo_shift = 32;
+    if (a.memo) {
+        int lg = 0;
+        while ((1 << lg) < memo_slots) ++lg;
+        VL_REQUIRE((1 << lg) == memo_slots && lg >= 1 && lg <= 24, "memo slots must be a power of two");
+        a.memo_shift = 32 - lg;
+    }
     a.n_rows = n_rows; a.n_vectors = n_vectors; a.n_nodes = n_nodes;
     a.dim = (int)dim; a.nchunks = (int)((dim + 3) / 4);
     a.n_visit = (int)n_visit; a.width = (int)width; a.m = (int)m;
@@ -275,7 +322,7 @@ VL_EXPORT int vl_gather_distances(const float *queries, int64_t n_rows, const fl
     if (n_rows == 0 || width == 0) return VL_OK;
     VL_REQUIRE(queries && vectors && ids && out, "null pointer");
     return vl_launch_expand(queries, n_rows, vectors, n_vectors, dim, ids, nullptr, 0, nullptr, 0,
-                            width, width, nullptr, out, nullptr, 0, 1, 0, 0, 0, (hipStream_t)stream);
+                            width, width, nullptr, out, nullptr, 0, 1, 0, 0, 0, nullptr, 0, (hipStream_t)stream);
 }
 
 VL_EXPORT int vl_search_from_seeds(const float *queries, int64_t n_rows, int64_t dim,
@@ -287,6 +334,6 @@ VL_EXPORT int vl_search_from_seeds(const float *queries, int64_t n_rows, int64_t
     if (n_rows == 0 || n_visit == 0 || width == 0) return VL_OK;
     VL_REQUIRE(queries && visit && beams && vectors && idx_out && dist_out, "null pointer");
     return vl_launch_expand(queries, n_rows, vectors, n_vectors, dim, nullptr, visit, n_visit, beams,
-                            n_nodes, width, n_visit * width, idx_out, dist_out, nullptr, 0, 1, 0, n_visit, 0,
+                            n_nodes, width, n_visit * width, idx_out, dist_out, nullptr, 0, 1, 0, n_visit, 0, nullptr, 0,
                             (hipStream_t)stream);
 }
