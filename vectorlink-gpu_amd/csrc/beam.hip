@@ -297,37 +297,65 @@ __device__ inline int block_compact(const uint64_t *src, int n, uint64_t *dst, P
     return run;
 }
 
+// Raise the batch-wide running maximum *slot to at least cnt.  Same-address
+// atomics from thousands of workgroups serialise in L2 and were the most
+// expensive part of the merge step, so they are kept for the rare case only:
+// a row that is at the largest fill any row can have (bound) publishes it with
+// a plain store - every such writer stores the same value and no atomicMax of a
+// smaller value can lower it - and any row skips the update when a late read
+// shows the slot is already there.
+__device__ inline void raise_running_max(int *slot, int cnt, int bound) {
+    if (__hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= cnt) return;
+    if (cnt >= bound) __hip_atomic_store(slot, cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else atomicMax(slot, cnt);
+}
+
+// Smallest key over the workgroup of each thread's `mine` (kPadKey = none).
+// red: 2 * kQueueWaves keys of LDS, used alternately so one barrier per call suffices.
+__device__ inline uint64_t block_min_key(uint64_t mine, uint64_t *red, int round) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int nw = blockDim.x / kWave;
+#pragma unroll
+    for (int h = kWave / 2; h >= 1; h >>= 1) {
+        uint64_t o = __shfl_xor((unsigned long long)mine, h);
+        mine = o < mine ? o : mine;
+    }
+    uint64_t *slot = red + (round & 1) * kQueueWaves;
+    if (lane == 0) slot[wave] = mine;
+    __syncthreads();
+    uint64_t m = slot[0];
+    for (int w = 1; w < nw; ++w) m = slot[w] < m ? slot[w] : m;
+    return m;
+}
+
 template <int THREADS>
 __global__ __launch_bounds__(THREADS) void beam_merge2_kernel(MergeArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int Pc = a.Pc;
-    uint64_t *ck = reinterpret_cast<uint64_t *>(smem);  // candidates, sorted
-    uint64_t *cc = ck + Pc;                             // filtered candidates
-    uint64_t *qa = cc + Pc;                             // search queue [0, L)
-    uint64_t *va = qa + a.L;                            // visit queue [Vt, VL)
+    uint64_t *raw = reinterpret_cast<uint64_t *>(smem);  // candidate keys as they arrive
+    uint64_t *uk = raw + Pc;                             // the candidates that can matter, then sorted
+    uint64_t *cc = uk + Pc;                              // filtered for one merge
+    uint64_t *qa = cc + Pc;                              // search queue [0, L)
+    uint64_t *va = qa + a.L;                             // visit queue [Vt, VL)
     int32_t *seen_a = reinterpret_cast<int32_t *>(va + a.VL);
     int32_t *seen_b = seen_a + a.E;
     int32_t *exl = seen_b + a.E;
+    uint8_t *fl = reinterpret_cast<uint8_t *>(exl + a.excl_cols);  // per candidate: bit0 wanted, bit1 rest
     __shared__ int wave_cnt[kQueueWaves];
+    __shared__ uint64_t red[2 * kQueueWaves];
     __shared__ int n_ex_s;
     __shared__ int32_t newv[kMaxVisit];
     __shared__ int n_new_s;
 
+    // Every global read of this workgroup is issued up front, before any of them
+    // is waited for: the control words, the candidates, both queues, the popped
+    // ids and the visited list (its fill is at most Vt ids per earlier iteration,
+    // so the row can be fetched without first waiting for the exact count).
     BeamCtrl *c = a.ctrl;
-    if (c->stop) return;
     const int t = a.iter;
     const int64_t row = blockIdx.x;
     const int lane = threadIdx.x & (kWave - 1);
-    int cnt = a.seen_count[row];
-    int *first_next = &c->first[(t + 1) & 1];
-    if (t >= 2 && c->first[(t - 1) & 1] >= a.E) {
-        if (threadIdx.x == 0) atomicMax(first_next, cnt);
-        return;
-    }
-    const int first = c->first[t & 1];
-    const bool seen_full = first >= a.E;
-    const bool checking = (t % a.readahead) == 0;
-
     int32_t *qi = a.q_ids + row * a.cap;
     float *qd = a.q_d + row * a.cap;
     int32_t *vi = a.v_ids + row * a.VL;
@@ -335,8 +363,23 @@ __global__ __launch_bounds__(THREADS) void beam_merge2_kernel(MergeArgs a) {
     const int32_t *ci = a.cand_ids + row * a.m;
     const float *cd = a.cand_d + row * a.m;
     const int nva = a.VL - a.Vt;
+    int *first_next = &c->first[(t + 1) & 1];
 
-    // ---- load -----------------------------------------------------------------
+    const int stop = c->stop;
+    const int first_prev = c->first[(t - 1) & 1];
+    const int first = c->first[t & 1];
+    int cnt = a.seen_count[row];
+    const int seen_bound = min(a.E, a.Vt * (t - 1));
+    for (int i = threadIdx.x; i < a.m; i += blockDim.x) raw[i] = vl_make_key(ci[i], cd[i]);
+    for (int i = threadIdx.x; i < a.L; i += blockDim.x) qa[i] = vl_make_key(qi[i], qd[i]);
+    for (int i = threadIdx.x; i < nva; i += blockDim.x) va[i] = vl_make_key(vi[a.Vt + i], vd[a.Vt + i]);
+    {
+        const int32_t *srow = a.seen + row * a.E;
+        for (int i = threadIdx.x; i < seen_bound; i += blockDim.x) seen_a[i] = srow[i];
+    }
+    // the ids popped at the start of this iteration (queue.py:87-95), before the row is rewritten
+    int32_t popped = VL_MAXINT;
+    if (threadIdx.x < kWave && (int)threadIdx.x < a.Vt) popped = vi[threadIdx.x];
     if (threadIdx.x == 0) {
         n_ex_s = a.excl ? a.excl_cols : 0;
         n_new_s = 0;
@@ -350,111 +393,152 @@ __global__ __launch_bounds__(THREADS) void beam_merge2_kernel(MergeArgs a) {
             if (e == VL_MAXINT) atomicMin(&n_ex_s, i);
         }
     }
-    for (int i = threadIdx.x; i < Pc; i += blockDim.x) ck[i] = i < a.m ? vl_make_key(ci[i], cd[i]) : kPadKey;
-    for (int i = threadIdx.x; i < a.L; i += blockDim.x) qa[i] = vl_make_key(qi[i], qd[i]);
-    for (int i = threadIdx.x; i < nva; i += blockDim.x) va[i] = vl_make_key(vi[a.Vt + i], vd[a.Vt + i]);
-    // the ids popped at the start of this iteration (queue.py:87-95), before the row is rewritten
-    int32_t popped = VL_MAXINT;
-    if (threadIdx.x < kWave && threadIdx.x < a.Vt) popped = vi[threadIdx.x];
-    if (!seen_full) {
-        const int32_t *srow = a.seen + row * a.E;
-        for (int i = threadIdx.x; i < cnt; i += blockDim.x) seen_a[i] = srow[i];
+    if (stop) return;
+    if (t >= 2 && first_prev >= a.E) {
+        // the visit queue is no longer fed: every candidate of this iteration is empty
+        if (threadIdx.x == 0) raise_running_max(first_next, cnt, min(a.E, a.Vt * t));
+        return;
     }
-    block_bitonic_sort(ck, Pc);
+    const bool seen_full = first >= a.E;
+    const bool checking = (t % a.readahead) == 0;
+    __syncthreads();
     const int n_ex = n_ex_s;
-    // real candidates sort before every empty pair and pad
-    const int n_real = key_lower_bound(ck, Pc, vl_make_key(VL_MAXINT, VL_MAXFLOAT));
 
-    // ---- search_queue.insert : ann.py:75-80 -------------------------------------
-    auto keep_search = [&](int i) -> bool {
-        uint64_t k = ck[i];
+    // ---- add_new_to_seen_ : utils.py:61-82 (does not depend on the candidates) ------
+    if (!seen_full) {
+        const int n_add = min(a.E - first, a.Vt);
+        if (threadIdx.x < kWave) {
+            const int j = threadIdx.x;
+            int32_t x = j < n_add ? popped : VL_MAXINT;
+            bool valid = j < n_add && x != VL_MAXINT && !sorted_contains(seen_a, cnt, x);
+            for (int i = 0; i < n_add; ++i) {
+                int32_t y = __shfl(popped, i);
+                if (i < j && y == x) valid = false;
+            }
+            uint64_t vm = __ballot(valid);
+            int rank = 0;
+            for (int i = 0; i < n_add; ++i) {
+                int32_t y = __shfl(popped, i);
+                if (((vm >> i) & 1) && y < x) ++rank;
+            }
+            if (valid) newv[rank] = x;
+            if (j == 0) n_new_s = __popcll(vm);
+        }
+        __syncthreads();
+        const int n_new = n_new_s;
+        for (int p = threadIdx.x; p < cnt; p += blockDim.x) {
+            int32_t v = seen_a[p];
+            int shift = 0;
+            for (int i = 0; i < n_new; ++i) shift += newv[i] < v;
+            seen_b[p + shift] = v;
+        }
+        if ((int)threadIdx.x < n_new)
+            seen_b[lower_bound(seen_a, cnt, newv[threadIdx.x]) + threadIdx.x] = newv[threadIdx.x];
+        __syncthreads();
+        cnt += n_new;
+        if (n_new) {
+            int32_t *srow = a.seen + row * a.E;
+            for (int i = threadIdx.x; i < cnt; i += blockDim.x) srow[i] = seen_b[i];
+        }
+        if (threadIdx.x == 0 && n_new) a.seen_count[row] = cnt;
+    }
+    if (threadIdx.x == 0) raise_running_max(first_next, cnt, min(a.E, a.Vt * t));
+
+    // ---- which candidates can matter at all -------------------------------------------
+    // search queue: only keys below its last slot can enter.  visit queue (VL slots, Vt of
+    // them just freed): every unvisited key below its last live slot, plus the Vt best
+    // distinct unvisited keys above it.  Everything else is dropped before the sort.
+    const uint64_t ws = qa[a.L - 1];
+    const uint64_t wv = nva > 0 ? va[nva - 1] : 0ull;
+    for (int i = threadIdx.x; i < a.m; i += blockDim.x) {
+        uint64_t k = raw[i];
         int32_t id = vl_key_id(k);
-        if (i > 0 && id == vl_key_id(ck[i - 1])) return false;   // neighbouring duplicate (kernels.py:314-349)
+        uint8_t f = 0;
+        if (id != VL_MAXINT) {
+            if (k < ws) f |= 1;
+            if (!seen_full && k != wv) {  // k == wv is the visit queue's own last slot again
+                bool unseen = !sorted_contains(seen_b, cnt, id);
+                if (unseen) f |= (k < wv) ? 1 : 2;
+            }
+        }
+        fl[i] = f;
+    }
+    uint64_t sel_max = 0ull;  // largest selected key among the "rest" candidates
+    if (!seen_full) {
+        uint64_t last = wv;
+        for (int r = 0; r < a.Vt; ++r) {
+            uint64_t mine = kPadKey;
+            for (int i = threadIdx.x; i < a.m; i += blockDim.x) {
+                uint64_t k = raw[i];
+                if ((fl[i] & 2) && k > last && k < mine) mine = k;
+            }
+            uint64_t mn = block_min_key(mine, red, r);
+            if (mn == kPadKey) break;
+            last = mn;
+            sel_max = mn;
+        }
+    }
+    __syncthreads();
+    auto wanted = [&](int i) -> bool {
+        uint8_t f = fl[i];
+        return (f & 1) || ((f & 2) && raw[i] <= sel_max);
+    };
+    const int n_u = block_compact(raw, a.m, uk, wanted, wave_cnt);
+    int Pu = 2;
+    while (Pu < n_u) Pu <<= 1;
+    for (int i = n_u + threadIdx.x; i < Pu; i += blockDim.x) uk[i] = kPadKey;
+    block_bitonic_sort(uk, Pu);
+
+    // ---- search_queue.insert : ann.py:75-80 -------------------------------------------
+    auto keep_search = [&](int i) -> bool {
+        uint64_t k = uk[i];
+        int32_t id = vl_key_id(k);
+        if (i > 0 && id == vl_key_id(uk[i - 1])) return false;   // neighbouring duplicate (kernels.py:314-349)
+        if (!(k < ws)) return false;
         for (int e = 0; e < n_ex; ++e)
             if (exl[e] == id) return false;                      // queue.py:52-53
         int p = key_lower_bound(qa, a.L, k);
         return !(p < a.L && qa[p] == k);                         // already queued
     };
-    const int n_s = block_compact(ck, n_real, cc, keep_search, wave_cnt);
+    const int n_s = block_compact(uk, n_u, cc, keep_search, wave_cnt);
     bool diff = false;
-    for (int i = threadIdx.x; i < a.L; i += blockDim.x) {
-        uint64_t k = qa[i];
-        int r = i + key_lower_bound(cc, n_s, k);
-        if (r < a.L) {
-            qi[r] = vl_key_id(k);
-            qd[r] = vl_key_dist(k);
+    if (n_s) {
+        for (int i = threadIdx.x; i < a.L; i += blockDim.x) {
+            uint64_t k = qa[i];
+            int r = i + key_lower_bound(cc, n_s, k);
+            if (r != i && r < a.L) {
+                qi[r] = vl_key_id(k);
+                qd[r] = vl_key_dist(k);
+            }
         }
-    }
-    for (int j = threadIdx.x; j < n_s; j += blockDim.x) {
-        uint64_t k = cc[j];
-        int r = j + key_lower_bound(qa, a.L, k);
-        if (r < a.L) {
-            qi[r] = vl_key_id(k);
-            qd[r] = vl_key_dist(k);
-            diff = true;  // a new id inside the first L slots: the row changed (queue.py:57-59)
+        for (int j = threadIdx.x; j < n_s; j += blockDim.x) {
+            uint64_t k = cc[j];
+            int r = j + key_lower_bound(qa, a.L, k);
+            if (r < a.L) {
+                qi[r] = vl_key_id(k);
+                qd[r] = vl_key_dist(k);
+                diff = true;  // a new id inside the first L slots: the row changed (queue.py:57-59)
+            }
         }
     }
     if (checking && __ballot(diff) && lane == 0) {
-        int *flag = &c->changed[(t / a.readahead) & 63];
-        if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) atomicOr(flag, 1);
+        int *flag = &c->changed[(t / a.readahead) & 63];  // every writer stores the same 1: no atomic needed
+        if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
+            __hip_atomic_store(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-
-    if (seen_full) {
-        if (threadIdx.x == 0) atomicMax(first_next, cnt);
-        return;
-    }
+    if (seen_full) return;
     __syncthreads();  // cc is reused below
 
-    // ---- add_new_to_seen_ : utils.py:61-82 ---------------------------------------
-    const int n_add = min(a.E - first, a.Vt);
-    if (threadIdx.x < kWave) {
-        const int j = threadIdx.x;
-        int32_t x = j < n_add ? popped : VL_MAXINT;
-        bool valid = j < n_add && x != VL_MAXINT && !sorted_contains(seen_a, cnt, x);
-        int rank = 0;
-        for (int i = 0; i < n_add; ++i) {
-            int32_t y = __shfl(popped, i);
-            if (i < j && y == x) valid = false;
-        }
-        uint64_t vm = __ballot(valid);
-        for (int i = 0; i < n_add; ++i) {
-            int32_t y = __shfl(popped, i);
-            if (((vm >> i) & 1) && y < x) ++rank;
-        }
-        if (valid) newv[rank] = x;
-        if (j == 0) n_new_s = __popcll(vm);
-    }
-    __syncthreads();
-    const int n_new = n_new_s;
-    for (int p = threadIdx.x; p < cnt; p += blockDim.x) {
-        int32_t v = seen_a[p];
-        int shift = 0;
-        for (int i = 0; i < n_new; ++i) shift += newv[i] < v;
-        seen_b[p + shift] = v;
-    }
-    if (threadIdx.x < n_new) seen_b[lower_bound(seen_a, cnt, newv[threadIdx.x]) + threadIdx.x] = newv[threadIdx.x];
-    __syncthreads();
-    cnt += n_new;
-    if (n_new) {
-        int32_t *srow = a.seen + row * a.E;
-        for (int i = threadIdx.x; i < cnt; i += blockDim.x) srow[i] = seen_b[i];
-    }
-    if (threadIdx.x == 0) {
-        a.seen_count[row] = cnt;
-        // the running maximum only grows: most rows find it already at their fill and skip the atomic
-        if (__hip_atomic_load(first_next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < cnt) atomicMax(first_next, cnt);
-    }
-
-    // ---- visit_queue.insert(candidates, exclude=seen) : ann.py:85-88 --------------
+    // ---- visit_queue.insert(candidates, exclude=seen) : ann.py:85-88 --------------------
     auto keep_visit = [&](int i) -> bool {
-        uint64_t k = ck[i];
+        uint64_t k = uk[i];
         int32_t id = vl_key_id(k);
-        if (i > 0 && id == vl_key_id(ck[i - 1])) return false;
+        if (i > 0 && id == vl_key_id(uk[i - 1])) return false;
         if (sorted_contains(seen_b, cnt, id)) return false;      // kernels.py:471-488
         int p = key_lower_bound(va, nva, k);
         return !(p < nva && va[p] == k);
     };
-    const int n_v = block_compact(ck, n_real, cc, keep_visit, wave_cnt);
+    const int n_v = block_compact(uk, n_u, cc, keep_visit, wave_cnt);
     for (int i = threadIdx.x; i < nva; i += blockDim.x) {
         uint64_t k = va[i];
         int r = i + key_lower_bound(cc, n_v, k);
@@ -592,14 +676,17 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
         const char *e = getenv("VL_BEAM_MERGE");
         return e && e[0] == 's';
     }();
-    static const int merge_threads = [] {
+    // threads per row of the merge step: small rows are latency bound and do better with
+    // more rows in flight per CU (measured: 128 wins at m=256, E=480; 256 wins at m=512, E=960)
+    static const int merge_threads_env = [] {
         const char *e = getenv("VL_BEAM_MERGE_THREADS");
-        return e ? atoi(e) : 256;
+        return e ? atoi(e) : 0;
     }();
+    const int merge_threads = merge_threads_env ? merge_threads_env : ((l.m + l.E + l.VL + p->queue_length) <= 1024 ? 128 : 256);
     const int Pmax = a.Ps > a.Pv ? a.Ps : a.Pv;
     const size_t smem = use_sort_merge
         ? (size_t)Pmax * 8 + (size_t)a.L * 4 + (size_t)a.E * 8 + (size_t)a.excl_cols * 4
-        : (size_t)a.Pc * 16 + (size_t)(a.L + a.VL) * 8 + (size_t)a.E * 8 + (size_t)a.excl_cols * 4;
+        : (size_t)a.Pc * 24 + (size_t)(a.L + a.VL) * 8 + (size_t)a.E * 8 + (size_t)a.excl_cols * 4 + (size_t)a.m + 16;
     VL_REQUIRE(smem <= 60 * 1024, "queues of this size need %zu bytes of LDS (limit 61440)", smem);
 
     const int R = (int)p->speculative_readahead;
