@@ -184,6 +184,23 @@ int vl_beam_profile(int enable, int reset, double *out);
 int vl_prune(const int32_t *beams, const float *dists, int64_t n, int64_t width,
              int32_t *beams_out, float *dists_out, void *stream);
 
+/* ---- rank-based graph optimisation ------------------------------------- */
+/* Detour-count re-ordering of every neighbour row and reverse-edge merge (the
+ * CAGRA optimisation).  No counterpart in the reference: its prune is vl_prune
+ * above and its reverse-edge collector is commented out (kernels.py:503-550).
+ * beams [n, width] holds rows ordered best first with distinct ids, VL_MAXINT
+ * for empty slots.  For the edge x->y at slot j a detour is a slot i < j of
+ * row x whose node lists y at a slot k < j; slots are re-ordered by (detours,
+ * slot) and cut to `degree`.  Then node y collects the sources x of edges
+ * x->y found in the first degree/2 slots of the cut rows, ordered by (slot,
+ * x), at most degree - degree/2 of them, and the final row of x is its first
+ * degree/2 edges, then its reverse edges not yet in the row (never x), then
+ * its remaining edges, cut to `degree`, padded with VL_MAXINT.
+ * out [n, degree] holds ids only; distances come from vl_gather_distances. */
+int64_t vl_optimize_graph_workspace_bytes(int64_t n, int64_t width, int64_t degree);
+int vl_optimize_graph(const int32_t *beams, int64_t n, int64_t width, int64_t degree,
+                      int32_t *out, void *workspace, int64_t workspace_bytes, void *stream);
+
 /* ---- exact k nearest neighbours on dense fp32 MFMA tiles -------------- */
 /* No counterpart in the reference (its recall is self-recall@1 only,
  * ann.py:235-259); used for ground truth recall@k.  ids_out/dists_out are

@@ -434,3 +434,50 @@ def test_dense_seeded_search():
     rec_circ = ann.recall_at_k(dev(q), 10, seeding="circulant")
     assert rec_dense > 0.9 and rec_dense == pytest.approx(ann.recall_at_k(dev(q), 10), abs=0.02)
     assert rec_dense >= rec_circ
+
+
+# ---------------------------------------------------------------- rank-based graph optimisation (addition)
+@pytest.mark.parametrize("n,w,d", [(40, 8, 4), (300, 12, 6), (1000, 64, 32), (700, 128, 64), (200, 6, 6), (50, 5, 1)])
+def test_optimize_graph(n, w, d):
+    say(f"optimize_graph n={n} w={w} d={d}")
+    from vectorlink_gpu.kernels import optimize_graph
+
+    rng = np.random.default_rng(n + w)
+    beams = np.stack([rng.choice([j for j in range(n) if j != i], w, replace=False) for i in range(n)]).astype(np.int32)
+    beams[rng.random((n, w)) < 0.05] = M
+    beams = np.stack([np.concatenate([r[r != M], r[r == M]]) for r in beams])
+    want = orc.optimize_graph(beams, d)
+    got = host(optimize_graph(dev(beams), d))
+    assert np.array_equal(got, want)
+
+
+def test_rank_pruned_build():
+    say("build with prune='rank'")
+    from vectorlink_gpu import ANN
+
+    rng = np.random.default_rng(31)
+    n, dim = 1200, 16
+    v = unit(rng, n, dim)
+    kw = dict(beam_size=8, beam_queue_factor=3, recall_search_queue_factor=2, batch_size=500, optimization_loops=2)
+    ann = ANN(dev(v), prune="rank", **kw)
+    # the oracle's version of the same pipeline: loops without pruning at full width, then optimize_graph
+    c = cfg(prune=False, **kw)
+    beams = orc.generate_circulant_beams(n, orc.primes(24))
+    d = orc.calculate_distances(v, beams)
+    for _ in range(2):
+        nb, nd = np.empty_like(beams), np.empty_like(d)
+        for s in range(0, n, 500):
+            e = min(s + 500, n)
+            q = orc.Queue(e - s, 24, 24 + 24 * 4)
+            q.insert(beams[s:e], d[s:e])
+            orc.closest_vectors(v[s:e], q, v, beams, c, orc.excluding_self(s, e))
+            nb[s:e], nd[s:e] = q.indices[:, :24], q.distances[:, :24]
+        beams, d = nb, nd
+        _, rec = orc.ann_calculate_recall(v, np.ascontiguousarray(beams[:, :8]), c, sample=v[:1000])
+        if rec == 1.0:
+            break
+    want = orc.optimize_graph(beams, 8)
+    assert np.array_equal(host(ann.beams), want)
+    real = want != M
+    wd = orc.calculate_distances(v, np.where(real, want, 0).astype(np.int32))
+    assert np.array_equal(bits(host(ann.distances)[real]), bits(wd[real]))

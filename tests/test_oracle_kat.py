@@ -328,3 +328,79 @@ def test_seen_add():
     # no column is free in every row any more -> None
     assert orc.add_new_to_seen_(seen, np.array([[20, 21], [22, 23]], np.int32)) is None
     assert seen.tolist() == [[3, 4, 5, 8, 9, 11], [1, 2, 7, 13, M, M]]
+
+
+# ---------------------------------------------------------------- rank prune / reverse merge (additions)
+def model_rank_prune(beams, degree):
+    n, w = beams.shape
+    out = np.full((n, degree), M, np.int32)
+    for x in range(n):
+        scored = []
+        for j in range(w):
+            y = beams[x, j]
+            if y == M:
+                continue
+            c = sum(1 for i in range(j) if beams[x, i] != M and y in beams[beams[x, i], :j].tolist())
+            scored.append((c, j, y))
+        scored.sort()
+        for o, (_, _, y) in enumerate(scored[:degree]):
+            out[x, o] = y
+    return out
+
+
+def model_reverse_merge(pruned, keep, rev_from):
+    n, d = pruned.shape
+    rev = {y: [] for y in range(n)}
+    for k, x in sorted((k, x) for x in range(n) for k in range(rev_from)):
+        y = pruned[x, k]
+        if y != M:
+            rev[int(y)].append((k, x))
+    out = np.full((n, d), M, np.int32)
+    for x in range(n):
+        row = [int(y) for y in pruned[x, :keep] if y != M]
+        for _, r in sorted(rev[x])[:d - keep]:
+            if r != x and r not in row and len(row) < d:
+                row.append(r)
+        for y in pruned[x, keep:]:
+            if y != M and int(y) not in row and len(row) < d:
+                row.append(int(y))
+        out[x, :len(row)] = row
+    return out
+
+
+def test_rank_prune_kat():
+    # 0 lists [1,2,3]; 1 lists 2 first: the edge 0->2 (slot 1) has the detour 0->1->2 (slot 0 of row 1 < 1)
+    beams = np.array([[1, 2, 3], [2, 0, 3], [3, 0, 1], [0, 1, 2]], np.int32)
+    got = orc.rank_prune(beams, 3)
+    # row 0: 1 (no slot before it), 2 (detour via 1), 3 (via 1? row 1[:2]=[2,0] no; via 2: row 2[:2]=[3,0] yes)
+    assert got[0].tolist() == [1, 2, 3]
+    beams = np.array([[1, 2, 3], [3, 2, 0], [0, 1, 3], [0, 1, 2]], np.int32)
+    # row 0: 2 has no detour (row 1[:1]=[3]); 3 has one (row 1[:2] holds 3) -> order unchanged, counts [0,0,1]
+    assert orc.rank_prune(beams, 2)[0].tolist() == [1, 2]
+    beams = np.array([[1, 3, 2], [3, 2, 0], [0, 1, 3], [0, 1, 2]], np.int32)
+    # row 0: slot1=3 detour via 1 (row 1[:1]=[3]) -> count 1; slot2=2: via 1 (row1[:2] has 2) -> 1, via 3 (row3[:2]=[0,1]) no
+    assert orc.rank_prune(beams, 3)[0].tolist() == [1, 3, 2]
+    beams = np.array([[1, 3, 2], [0, 2, 3], [0, 1, 3], [0, 1, 2]], np.int32)
+    # row 0: 3 -> none (row1[:1]=[0]); 2 -> via 1 (row1[:2]=[0,2]) -> counts [0,0,1]
+    assert orc.rank_prune(beams, 3)[0].tolist() == [1, 3, 2]
+    beams = np.array([[1, 2, 3], [3, 0, 2], [0, 1, 3], [0, 1, 2]], np.int32)
+    # row 0: 2 -> none (row1[:1]=[3]); 3 -> via 1 (row1[:2]=[3,0]) -> counts [0,0,1]; with M holes
+    beams[0, 1] = M
+    assert orc.rank_prune(beams, 3)[0].tolist() == [1, 3, M]
+
+
+def test_rank_prune_and_reverse_merge_against_models():
+    rng = np.random.default_rng(30)
+    for n, w, d in [(40, 8, 4), (60, 12, 6), (25, 6, 6)]:
+        beams = np.stack([rng.choice([j for j in range(n) if j != i], w, replace=False) for i in range(n)]).astype(np.int32)
+        beams[rng.random((n, w)) < 0.08] = M
+        beams = np.stack([np.concatenate([r[r != M], r[r == M]]) for r in beams])  # empties last, as after a sort
+        got = orc.rank_prune(beams, d)
+        assert np.array_equal(got, model_rank_prune(beams, d))
+        for keep, rev_from in [(d // 2, d // 2), (1, d), (d, 2)]:
+            merged = orc.reverse_merge(got, keep, rev_from)
+            assert np.array_equal(merged, model_reverse_merge(got, keep, rev_from))
+            for x in range(n):
+                real = merged[x][merged[x] != M]
+                assert len(set(real.tolist())) == len(real) and x not in real.tolist()
+                assert merged[x, :keep].tolist()[:int((got[x, :keep] != M).sum())] == got[x, :keep][got[x, :keep] != M].tolist()

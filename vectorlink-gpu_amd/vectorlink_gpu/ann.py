@@ -14,7 +14,7 @@ from torch import Tensor
 
 from . import _native as nv
 from .constants import DEVICE, MAXFLOAT, MAXINT
-from .kernels import calculate_distances, gather_distances, knn_exact, prune_, search_from_seeds
+from .kernels import calculate_distances, gather_distances, knn_exact, optimize_graph, prune_, search_from_seeds
 from .log import log_time
 from .queue import Queue
 from .utils import add_new_to_seen_, generate_circulant_beams, generate_queue_circulants, primes
@@ -175,7 +175,7 @@ class GraphBuild:
         self.finished = True
 
     def _finish_loop(self, next_beams: Tensor, next_beam_distances: Tensor) -> float:
-        if self.config["prune"]:  # ann.py:171-177
+        if self.config["prune"] is True:  # ann.py:171-177 (prune="rank" thins nothing between loops)
             (self.beams, self.distances) = prune_(next_beams, next_beam_distances)
         else:
             (self.beams, self.distances) = (next_beams, next_beam_distances)
@@ -185,6 +185,10 @@ class GraphBuild:
         return recall
 
     def result(self) -> Tuple[Tensor, Tensor]:
+        if self.config["prune"] == "rank":
+            # addition: cut the full-width table to beam_size by detour count and merge reverse edges
+            ids = optimize_graph(self.beams, self.beam_size)
+            return (ids, gather_distances(self.vectors, self.vectors, ids))
         out_distances = self.beam_distances if self.stale else self.distances  # ann.py:190-193
         return (self.beams.narrow_copy(1, 0, self.beam_size), out_distances.narrow_copy(1, 0, self.beam_size))
 
@@ -311,7 +315,11 @@ class ANN:
     ):
         """seeding / entry_points are additions: "circulant" seeds searches as the
         reference does; "dense" seeds them from the nearest of `entry_points`
-        evenly spread vectors (see dense_search_queue)."""
+        evenly spread vectors (see dense_search_queue).  prune also accepts
+        "rank": no pruning between loops, and the final cut from the build queue
+        width to beam_size is done by detour count with reverse edges merged in
+        (kernels.optimize_graph) instead of keeping the first beam_size columns."""
+        assert prune in (True, False, "rank")
         assert vectors.dim() == 2 and vectors.dtype == torch.float32
         assert seeding in ("circulant", "dense")
         self.seeding = seeding

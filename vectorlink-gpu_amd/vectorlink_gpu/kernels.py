@@ -170,3 +170,19 @@ def knn_exact(queries: Tensor, vectors: Tensor, k: int) -> Tuple[Tensor, Tensor]
     nv.check(nv.lib().vl_knn_exact(nv.ptr(queries), nq, nv.ptr(vectors), vectors.size(0), dim, k, nv.ptr(ids),
                                    nv.ptr(dists), nv.ptr(ws), ws.numel(), nv.stream()))
     return (ids, dists)
+
+
+def optimize_graph(beams: Tensor, degree: int) -> Tensor:
+    """Rank-based graph optimisation (not in the reference): re-order every row of
+    `beams` ([N, W], best first, MAXINT = empty) by the number of two-hop detours
+    of each edge, cut to `degree`, and merge in reverse edges.  Returns ids
+    [N, degree]; see include/vlgpu.h for the exact rule."""
+    _check_ids(beams, "beams")
+    nv.require_gpu(beams)
+    (n, width) = beams.size()
+    need = nv.check(nv.lib().vl_optimize_graph_workspace_bytes(n, width, degree))
+    ws = torch.empty(max(need, 256), dtype=torch.uint8, device=beams.device)
+    out = torch.empty((n, degree), dtype=torch.int32, device=beams.device)
+    nv.check(nv.lib().vl_optimize_graph(nv.ptr(beams), n, width, degree, nv.ptr(out), nv.ptr(ws), ws.numel(),
+                                        nv.stream()))
+    return out
