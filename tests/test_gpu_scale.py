@@ -1,0 +1,130 @@
+"""GPU checks at the full sizes of the benchmark workloads (1M x 128 and
+1M x 768), through properties that do not need the CPU oracle to run at that
+scale: ordering, membership, distances recomputed from ids, float64 samples,
+round trips, determinism - plus a small batch at full scale replayed on the
+oracle for exact ids."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+M = orc.MAXINT
+DEV = "cuda"
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+@pytest.fixture(scope="module")
+def mix128():
+    from vectorlink_gpu import synthetic
+
+    base, q, w = synthetic.make("mix-1m-128")
+    return base, q, w
+
+
+def test_build_1m_x_128_properties(mix128):
+    say("full build 1M x 128")
+    from vectorlink_gpu import ANN, synthetic
+    from vectorlink_gpu.kernels import gather_distances, knn_exact
+
+    base, q, w = mix128
+    v = base.to(DEV)
+    ann = ANN(v, **synthetic.ann_kwargs(w))
+    n, deg = ann.beams.shape
+    assert (n, deg) == (1_000_000, 32) and ann.distances.shape == (n, deg)
+    ids, d = ann.beams, ann.distances
+    real = ids != M
+    assert bool(real[:, 0].all())
+    assert bool(((ids >= 0) & (ids < n))[real].all())
+    rows = torch.arange(n, device=DEV, dtype=torch.int32).unsqueeze(1).expand(n, deg)
+    assert not bool((ids == rows)[real].any())                       # no self edges
+    assert bool((d[:, 1:] >= d[:, :-1]).all())                        # rows ordered by distance
+    srt = ids.sort(dim=1).values
+    assert not bool(((srt[:, 1:] == srt[:, :-1]) & (srt[:, 1:] != M)).any())  # distinct ids per row
+    assert bool((d[~real] == torch.tensor(3.4028e37, device=DEV)).all())
+    # the distances are the distances of the ids: recomputed bit for bit, and against float64 on a sample
+    again = gather_distances(v, v, ids)
+    assert torch.equal(again, d)
+    sample = torch.randint(0, n, (512,), generator=torch.Generator().manual_seed(0))
+    vs = base[sample].double()
+    nb = base[ids[sample.to(DEV)].cpu().long()].double()              # [512, deg, dim]
+    ref = ((1 - (vs.unsqueeze(1) * nb).sum(2)) / 2).clamp(0, 1)
+    assert torch.allclose(d[sample.to(DEV)].cpu().double(), ref, rtol=1e-5, atol=1e-6)
+    # graph quality and search
+    t11, _ = knn_exact(v[:1024].contiguous(), v, 11)
+    hits = (ids[:1024, :, None] == t11[:, None, 1:11]).any(dim=1).sum().item()
+    assert hits / (1024 * 10) > 0.7
+    qd = q[:2000].to(DEV)
+    r1 = ann.search(qd, seeding="dense")
+    r2 = ann.search(qd, seeding="dense")
+    assert torch.equal(r1.indices[:, :r1.length], r2.indices[:, :r2.length])      # deterministic
+    assert bool((r1.distances[:, 1:r1.length] >= r1.distances[:, :r1.length - 1]).all())
+    truth, td = knn_exact(qd, v, 10)
+    found = r1.indices[:, :10]
+    recall = (found.unsqueeze(2) == truth.unsqueeze(1)).any(dim=2).sum().item() / truth.numel()
+    assert recall > 0.75
+    # what search returns are real distances of real ids
+    fd = gather_distances(qd, v, found.contiguous())
+    assert torch.equal(fd, r1.distances[:, :10])
+    # resume from the stored graph (ann.py:391-396): same distances, same answers
+    again = ANN(v, beams=ann.beams, **synthetic.ann_kwargs(w))
+    assert torch.equal(again.distances, d)
+    r3 = again.search(qd, seeding="dense")
+    assert torch.equal(r3.indices[:, :r3.length], r1.indices[:, :r1.length])
+
+
+def test_1m_x_768_distances_knn_and_one_batch_on_the_oracle():
+    say("1M x 768: distances, exact kNN, one small batch against the oracle")
+    from vectorlink_gpu import synthetic
+    from vectorlink_gpu.ann import closest_vectors, excluding_self
+    from vectorlink_gpu.kernels import calculate_distances, knn_exact
+    from vectorlink_gpu.queue import Queue
+    from vectorlink_gpu.utils import generate_circulant_beams, primes
+
+    base, q, w = synthetic.make("mix-1m-768")
+    n, dim = base.shape
+    v = base.to(DEV)
+    ql = w["beam_size"] * w["beam_queue_factor"]
+    beams = generate_circulant_beams(n, primes(ql))
+    d = calculate_distances(v, beams)
+    assert bool(((d >= 0) & (d <= 1)).all())
+    # closed form of the circulant table and float64 distances on a sample of rows
+    sample = torch.tensor([0, 1, 777_777, n - 1])
+    p = torch.from_numpy(orc.primes(ql).astype(np.int64))
+    want_ids = (sample.unsqueeze(1) + p.unsqueeze(0)) % n
+    assert torch.equal(beams[sample.to(DEV)].cpu().long(), want_ids)
+    ref = ((1 - (base[sample].double().unsqueeze(1) * base[want_ids].double()).sum(2)) / 2).clamp(0, 1)
+    assert torch.allclose(d[sample.to(DEV)].cpu().double(), ref, rtol=1e-5, atol=1e-6)
+    # symmetry d(a, b) == d(b, a), bit for bit, through the two operand roles
+    a, b = 12_345, int(want_ids[0, 5])
+    from vectorlink_gpu.kernels import gather_distances
+    dab = gather_distances(v[a:a + 1].contiguous(), v, torch.tensor([[b]], dtype=torch.int32, device=DEV))
+    dba = gather_distances(v[b:b + 1].contiguous(), v, torch.tensor([[a]], dtype=torch.int32, device=DEV))
+    assert torch.equal(dab, dba)
+    # exact kNN against a float64 brute force for a few queries
+    qd = q[:8].to(DEV)
+    gi, gd = knn_exact(qd, v, 10)
+    full = ((1 - q[:8].double() @ base.double().t()) / 2).clamp(0, 1)
+    wd, wi = full.topk(10, dim=1, largest=False)
+    assert torch.allclose(gd.cpu().double(), wd, rtol=1e-5, atol=1e-6)
+    assert (gi.cpu().long() == wi).float().mean() > 0.95
+    # one batch of 24 rows of the first optimisation loop, replayed on the CPU oracle: exact ids and distances
+    rows = 24
+    cfg = dict(orc.DEFAULT_CONFIG)
+    cfg.update(synthetic.ann_kwargs(w))
+    gq = Queue(rows, ql, ql + ql * 4)
+    gq.insert(beams[:rows], d[:rows])
+    t_gpu = closest_vectors(v[:rows], gq, v, beams, cfg, excluding_self(0, rows))
+    vn = base.numpy()
+    ob = orc.generate_circulant_beams(n, orc.primes(ql))
+    oq = orc.Queue(rows, ql, ql + ql * 4)
+    oq.insert(ob[:rows], orc.gather_distances(vn[:rows], vn, ob[:rows]))
+    t_cpu = orc.closest_vectors(vn[:rows], oq, vn, ob, cfg, orc.excluding_self(0, rows))
+    assert t_gpu == t_cpu
+    assert np.array_equal(gq.indices[:, :ql].cpu().numpy(), oq.indices[:, :ql])
+    assert np.array_equal(gq.distances[:, :ql].cpu().numpy().view(np.uint32), oq.distances[:, :ql].view(np.uint32))
