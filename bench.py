@@ -28,10 +28,12 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
-# Bytes moved past L2 per expand launch, from two rocprofv3 --pmc runs (FETCH_SIZE x 2.0 after calibration
-# against a 1 GiB copy, + WRITE_SIZE x 1.0); profiles/expand_kernel_mix-1m-768_hbm_traffic.txt holds the runs.
+# Bytes moved past L2 per expand launch, from two rocprofv3 --pmc runs over the first 104 build steps
+# (FETCH_SIZE x 2.0 after calibration against a 1 GiB copy, + WRITE_SIZE x 1.0); the same runs' algorithmic
+# bytes per launch are given beside it.  profiles/expand_kernel_mix-1m-768_hbm_traffic.txt holds the runs.
 # Workloads without a recorded counter run report null.
-TRAFFIC_BYTES_PER_LAUNCH = {"mix-1m-768": 14.87e9}
+TRAFFIC = {"mix-1m-768": dict(bytes_per_launch=12.36e9, algorithmic_bytes_per_launch_in_that_run=12.03e9,
+                              scope="first 104 build steps (25,605 launches)")}
 
 
 def log(*a):
@@ -166,7 +168,8 @@ def main():
                  if prof["expand_ms"] > 0 else 0.0)
     roofline = dict(bound="hbm", kernel="expand_kernel (gathered cosine distances of the beam search)",
                     achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
-                    traffic=TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
+                    traffic=(TRAFFIC.get(args.workload) or {}).get("bytes_per_launch"),
+                    traffic_detail=TRAFFIC.get(args.workload),
                     launches=int(prof["expand_launches"]), avg_launch_ms=prof["expand_ms"] / launches,
                     algorithmic_bytes_per_launch=algo_bytes / launches,
                     reference_equivalent_gbs=effective,
