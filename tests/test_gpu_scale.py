@@ -128,3 +128,51 @@ def test_1m_x_768_distances_knn_and_one_batch_on_the_oracle():
     assert t_gpu == t_cpu
     assert np.array_equal(gq.indices[:, :ql].cpu().numpy(), oq.indices[:, :ql])
     assert np.array_equal(gq.distances[:, :ql].cpu().numpy().view(np.uint32), oq.distances[:, :ql].view(np.uint32))
+
+
+def test_offsets_beyond_2_to_31_elements():
+    """N x D above 2^31 elements (the shape class of the 20M x 384 and 10M x 1536 workloads):
+    every row offset must be computed in 64 bits."""
+    say("2.2M x 1024: 64-bit offsets")
+    from vectorlink_gpu.ann import closest_vectors, excluding_self
+    from vectorlink_gpu.kernels import calculate_distances, gather_distances, knn_exact
+    from vectorlink_gpu.queue import Queue
+    from vectorlink_gpu.utils import generate_circulant_beams, primes
+
+    n, dim = 2_200_000, 1024
+    assert n * dim > 2**31
+    g = torch.Generator(device=DEV).manual_seed(5)
+    v = torch.empty((n, dim), dtype=torch.float32, device=DEV)
+    for s in range(0, n, 200_000):
+        e = min(n, s + 200_000)
+        v[s:e] = torch.nn.functional.normalize(torch.randn((e - s, dim), generator=g, device=DEV), dim=1)
+    hi = n - 4096
+    # gathered distances between rows at the far end, against float64 on the device
+    rows = torch.arange(hi, hi + 512, device=DEV)
+    ids = torch.randint(hi, n, (512, 33), generator=g, device=DEV).to(torch.int32)
+    got = gather_distances(v[hi:hi + 512], v, ids)
+    ref = ((1 - (v[rows].double().unsqueeze(1) * v[ids.long()].double()).sum(2)) / 2).clamp(0, 1)
+    assert torch.allclose(got.double(), ref, rtol=1e-5, atol=1e-6)
+    # exact kNN: a query that is a copy of a far row must come back first at distance ~0
+    q = v[torch.tensor([n - 1, n - 77, 5], device=DEV)].contiguous()
+    ki, kd = knn_exact(q, v, 4)
+    assert ki[:, 0].tolist() == [n - 1, n - 77, 5] and float(kd[:, 0].max()) < 1e-6
+    full = ((1 - q.double() @ v[hi:].double().t()) / 2).clamp(0, 1)   # the far block alone bounds the answer
+    assert bool((kd[:, 1].double() <= full.topk(2, dim=1, largest=False).values[:, 1] + 1e-6).all())
+    # one beam-search batch over the last rows: ordered, self excluded, distances belong to the ids
+    cfg = dict(orc.DEFAULT_CONFIG)
+    cfg.update(beam_size=16, beam_queue_factor=2)
+    ql = 32
+    beams = generate_circulant_beams(n, primes(ql))
+    d = calculate_distances(v, beams)
+    s0, e0 = n - 1000, n
+    gq = Queue(e0 - s0, ql, ql + ql * 4)
+    gq.insert(beams[s0:e0], d[s0:e0])
+    t = closest_vectors(v[s0:e0], gq, v, beams, cfg, excluding_self(s0, e0))
+    assert t > 0 and t % 5 == 0
+    qi, qd = gq.indices[:, :ql], gq.distances[:, :ql]
+    assert bool((qd[:, 1:] >= qd[:, :-1]).all()) and bool((qi != M).all())
+    own = torch.arange(s0, e0, device=DEV, dtype=torch.int32).unsqueeze(1)
+    assert not bool((qi == own).any())
+    assert torch.equal(gather_distances(v[s0:e0], v, qi.contiguous()), qd)
+    assert bool((qd[:, 0] <= d[s0:e0].min(dim=1).values).all())       # never worse than the seeds
