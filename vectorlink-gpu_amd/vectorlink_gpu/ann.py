@@ -312,6 +312,7 @@ class ANN:
         distances: Optional[Tensor] = None,
         seeding: str = "circulant",
         entry_points: int = 32_768,
+        keep_queues: bool = False,
     ):
         """seeding / entry_points are additions: "circulant" seeds searches as the
         reference does; "dense" seeds them from the nearest of `entry_points`
@@ -325,6 +326,7 @@ class ANN:
         self.seeding = seeding
         self.entry_points = entry_points
         self._entry = None
+        self._queues = None
         (count, dim) = vectors.size()
         self.configuration: Dict = {
             "prune": prune,
@@ -349,14 +351,69 @@ class ANN:
             else:
                 self.distances = distances.to(self.vectors.device).contiguous()
         else:
-            self.build_stats: list = []
-            (self.beams, self.distances) = generate_ann(self.vectors, self.configuration, stats=self.build_stats)
+            build = GraphBuild(self.vectors, self.configuration)
+            for _ in build.steps():
+                pass
+            self.build_stats: list = build.stats
+            (self.beams, self.distances) = build.result()
+            if keep_queues:
+                width = build.beams.size(1)
+                self._queues = Queue(count, width, width + 1, device=self.vectors.device)
+                self._queues.indices[:, :width].copy_(build.beams)
+                self._queues.distances[:, :width].copy_(build.distances)
         torch.cuda.synchronize(self.vectors.device)
         wall_end = time.time()
         self.log = self.configuration.copy()
         self.log["total_time"] = wall_end - wall_start
         self.log["vector_count"] = count
         self.log["vector_dimension"] = dim
+
+    @classmethod
+    def load_from_dataframe(cls, dataframe, device=DEVICE, **kwargs) -> "ANN":
+        """reference ann.py:408-454: `dataframe` has the columns vector_id, embedding and
+        beams and optionally distances; rows are taken in vector_id order.  Accepts a
+        pyarrow Table or anything with DataFusion's `to_arrow_table()`."""
+        import pyarrow as pa
+        import pyarrow.compute as pc
+
+        from .datafusion import dataframe_to_tensor
+
+        table = dataframe.to_arrow_table() if hasattr(dataframe, "to_arrow_table") else dataframe
+        assert isinstance(table, pa.Table), "expected a pyarrow Table or a DataFusion DataFrame"
+        names = table.schema.names
+        assert "embedding" in names and "beams" in names
+        if "vector_id" in names:
+            table = table.take(pc.sort_indices(table, sort_keys=[("vector_id", "ascending")]))
+        count = table.num_rows
+
+        def width(name):
+            t = table.schema.field(name).type
+            if pa.types.is_fixed_size_list(t):
+                return t.list_size
+            return len(table.column(name)[0]) if count else 0
+
+        vectors = torch.empty((count, width("embedding")), dtype=torch.float32, device=device)
+        dataframe_to_tensor(table, vectors, "embedding")
+        beams = torch.empty((count, width("beams")), dtype=torch.int32, device=device)
+        dataframe_to_tensor(table, beams, "beams")
+        distances = None
+        if "distances" in names:
+            distances = torch.empty((count, beams.size(1)), dtype=torch.float32, device=device)
+            dataframe_to_tensor(table, distances, "distances")
+        return cls(vectors, beam_size=beams.size(1), beams=beams, distances=distances, **kwargs)
+
+    def to_arrow(self):
+        """The index as a pyarrow Table with the columns load_from_dataframe reads."""
+        import pyarrow as pa
+
+        from .datafusion import tensor_to_arrow
+
+        return pa.table({
+            "vector_id": pa.array(range(self.vectors.size(0)), type=pa.int32()),
+            "embedding": tensor_to_arrow(self.vectors),
+            "beams": tensor_to_arrow(self.beams),
+            "distances": tensor_to_arrow(self.distances),
+        })
 
     def recall(self, sample_size: int = 1000) -> Tuple[float, float]:
         """reference ann.py:456-464"""
@@ -366,8 +423,11 @@ class ANN:
         return ann_calculate_recall(self.vectors, self.beams, self.configuration, sample)
 
     def clusters(self):
-        """reference ann.py:466-467 (a stub there as well)"""
-        return None
+        """reference ann.py:466-467 is a stub (`pass`); its README says "returns all search
+        queues".  Here: the search queues the build ended with, one per vector at the
+        build queue width, as a Queue - when the index was built with keep_queues=True;
+        otherwise None, like the reference."""
+        return self._queues
 
     def _entry_tables(self):
         if self._entry is None:
