@@ -16,6 +16,7 @@
 // for progress (ann.py:68,90-91).
 #include "beam_ctrl.h"
 #include "rowsort.h"
+#include "dist_device.h"
 #include <stdlib.h>
 
 int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors, int64_t n_vectors,
@@ -329,9 +330,10 @@ __device__ inline uint64_t block_min_key(uint64_t mine, uint64_t *red, int round
     return m;
 }
 
-template <int THREADS>
-__global__ __launch_bounds__(THREADS) void beam_merge2_kernel(MergeArgs a) {
-    extern __shared__ __align__(16) unsigned char smem[];
+// FUSED: the candidates of this row are already in LDS (ids at uk, distances behind them,
+// written by the expand phase of the same workgroup) and the loop state has been checked.
+template <int THREADS, bool FUSED>
+__device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *smem) {
     const int Pc = a.Pc;
     uint64_t *raw = reinterpret_cast<uint64_t *>(smem);  // candidate keys as they arrive
     uint64_t *uk = raw + Pc;                             // the candidates that can matter, then sorted
@@ -365,12 +367,18 @@ __global__ __launch_bounds__(THREADS) void beam_merge2_kernel(MergeArgs a) {
     const int nva = a.VL - a.Vt;
     int *first_next = &c->first[(t + 1) & 1];
 
-    const int stop = c->stop;
-    const int first_prev = c->first[(t - 1) & 1];
+    const int stop = FUSED ? 0 : c->stop;
+    const int first_prev = FUSED ? 0 : c->first[(t - 1) & 1];
     const int first = c->first[t & 1];
     int cnt = a.seen_count[row];
     const int seen_bound = min(a.E, a.Vt * (t - 1));
-    for (int i = threadIdx.x; i < a.m; i += blockDim.x) raw[i] = vl_make_key(ci[i], cd[i]);
+    if constexpr (FUSED) {
+        const int32_t *li = reinterpret_cast<const int32_t *>(uk);
+        const float *ld = reinterpret_cast<const float *>(li + a.m);
+        for (int i = threadIdx.x; i < a.m; i += blockDim.x) raw[i] = vl_make_key(li[i], ld[i]);
+    } else {
+        for (int i = threadIdx.x; i < a.m; i += blockDim.x) raw[i] = vl_make_key(ci[i], cd[i]);
+    }
     for (int i = threadIdx.x; i < a.L; i += blockDim.x) qa[i] = vl_make_key(qi[i], qd[i]);
     for (int i = threadIdx.x; i < nva; i += blockDim.x) va[i] = vl_make_key(vi[a.Vt + i], vd[a.Vt + i]);
     {
@@ -394,7 +402,7 @@ __global__ __launch_bounds__(THREADS) void beam_merge2_kernel(MergeArgs a) {
         }
     }
     if (stop) return;
-    if (t >= 2 && first_prev >= a.E) {
+    if (!FUSED && t >= 2 && first_prev >= a.E) {
         // the visit queue is no longer fed: every candidate of this iteration is empty
         if (threadIdx.x == 0) raise_running_max(first_next, cnt, min(a.E, a.Vt * t));
         return;
@@ -561,6 +569,117 @@ __global__ __launch_bounds__(THREADS) void beam_merge2_kernel(MergeArgs a) {
     }
 }
 
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void beam_merge2_kernel(MergeArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    merge_row<THREADS, false>(a, smem);
+}
+
+// ---- one launch per iteration -------------------------------------------------
+// The expand phase (HBM bound) and the merge phase (LDS / latency bound) of one
+// row run in the same workgroup, so on every CU some workgroups stream candidate
+// rows while others merge: the merge time hides behind the memory traffic, the
+// candidate ids and distances never leave LDS, and an iteration is one launch.
+struct StepArgs {
+    MergeArgs m;
+    const float *queries;
+    const float *vectors;
+    const int32_t *beams;
+    int64_t n_vectors;
+    int dim, nchunks, width;
+    uint64_t *memo;
+    int memo_shift;
+    int count_evals;
+};
+
+template <int CPL, int LPR, int U, bool GENERIC, int THREADS>
+__global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const MergeArgs &a = s.m;
+    BeamCtrl *c = a.ctrl;
+    const int t = a.iter;
+    const int gate = beam_gate(c, t, a.readahead, a.E, blockIdx.x == 0 && threadIdx.x == 0);
+    if (gate == 2) return;
+    const int64_t row = blockIdx.x;
+    if (gate == 1) {
+        // the visit queue is no longer fed: every candidate of this iteration is empty
+        if (threadIdx.x == 0) raise_running_max(&c->first[(t + 1) & 1], a.seen_count[row], min(a.E, a.Vt * t));
+        return;
+    }
+    // ---- expand: ann.py:69-73 (pop the visit heads, gather their neighbour lists, distances) ----
+    uint64_t *uk = reinterpret_cast<uint64_t *>(smem) + a.Pc;
+    int32_t *li = reinterpret_cast<int32_t *>(uk);
+    float *ld = reinterpret_cast<float *>(li + a.m);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int32_t *visit = a.v_ids + row * a.VL;
+    const float *q_row = s.queries + row * s.dim;
+    uint64_t *memo_row = s.memo ? s.memo + ((uint64_t)row << (32 - s.memo_shift)) : nullptr;
+    for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
+        const int slot = c0 + lane;
+        const bool has = slot < a.m;
+        int32_t id = VL_MAXINT;
+        if (has) {
+            int sidx = slot / s.width, k = slot - sidx * s.width;
+            int32_t node = visit[sidx];
+            if (node != VL_MAXINT && (uint32_t)node < (uint64_t)s.n_vectors) id = s.beams[(int64_t)node * s.width + k];
+        }
+        bool ok = has && id != VL_MAXINT && id >= 0 && (int64_t)id < s.n_vectors;
+        if (has) {
+            li[slot] = ok ? id : VL_MAXINT;
+            if (!ok) ld[slot] = VL_MAXFLOAT;
+        }
+        if (s.count_evals) {
+            uint64_t wm = __ballot(ok);
+            if (lane == 0 && wm) atomicAdd(&c->wanted[blockIdx.x & 63], (unsigned long long)__popcll(wm));
+        }
+        if (memo_row && ok) {
+            uint64_t e = memo_row[memo_hash(id, s.memo_shift)];
+            if ((int32_t)(uint32_t)e == id) {
+                ld[slot] = __builtin_bit_cast(float, (uint32_t)(e >> 32));
+                ok = false;
+            }
+        }
+        if (s.count_evals) {
+            uint64_t okm = __ballot(ok);
+            if (lane == 0 && okm) atomicAdd(&c->evals[blockIdx.x & 63], (unsigned long long)__popcll(okm));
+        }
+        if constexpr (GENERIC)
+            wave_distances_generic(q_row, s.vectors, s.dim, s.nchunks, id, ok, ld + c0, memo_row, s.memo_shift);
+        else
+            wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, id, ok, ld + c0, memo_row, s.memo_shift);
+    }
+    __syncthreads();
+    // ---- merge: ann.py:75-88 ----
+    merge_row<THREADS, true>(a, smem);
+}
+
+template <int CPL, int LPR, int U, bool GENERIC>
+void launch_step(const StepArgs &s, int threads, size_t smem, hipStream_t st) {
+    dim3 grid((unsigned)s.m.n_rows);
+    if (threads == 128)
+        hipLaunchKernelGGL((beam_step_kernel<CPL, LPR, U, GENERIC, 128>), grid, dim3(128), smem, st, s);
+    else
+        hipLaunchKernelGGL((beam_step_kernel<CPL, LPR, U, GENERIC, 256>), grid, dim3(256), smem, st, s);
+}
+
+int launch_step_by_dim(const StepArgs &s, bool aligned, int threads, size_t smem, hipStream_t st) {
+    const int nchunks = s.nchunks;
+    if (!aligned || nchunks > 512) launch_step<1, 64, 1, true>(s, threads, smem, st);
+    else if (nchunks <= 16) launch_step<1, 16, 8, false>(s, threads, smem, st);
+    else if (nchunks <= 32) launch_step<1, 32, 8, false>(s, threads, smem, st);
+    else if (nchunks <= 64) launch_step<1, 64, 8, false>(s, threads, smem, st);
+    else if (nchunks <= 128) launch_step<2, 64, 8, false>(s, threads, smem, st);
+    else if (nchunks <= 192) launch_step<3, 64, 4, false>(s, threads, smem, st);
+    else if (nchunks <= 256) launch_step<4, 64, 4, false>(s, threads, smem, st);
+    else if (nchunks <= 320) launch_step<5, 64, 2, false>(s, threads, smem, st);
+    else if (nchunks <= 384) launch_step<6, 64, 2, false>(s, threads, smem, st);
+    else if (nchunks <= 448) launch_step<7, 64, 2, false>(s, threads, smem, st);
+    else launch_step<8, 64, 2, false>(s, threads, smem, st);
+    VL_LAUNCH_CHECK("beam_step_kernel");
+    return VL_OK;
+}
+
 struct BeamLayout {
     int64_t m, VL, Vt, E, head;
     int64_t off_cand_ids, off_cand_d, off_v_ids, off_v_d, off_seen, off_seen_count, off_ctrl, off_memo, total;
@@ -689,8 +808,27 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
         : (size_t)a.Pc * 24 + (size_t)(a.L + a.VL) * 8 + (size_t)a.E * 8 + (size_t)a.excl_cols * 4 + (size_t)a.m + 16;
     VL_REQUIRE(smem <= 60 * 1024, "queues of this size need %zu bytes of LDS (limit 61440)", smem);
 
+    // VL_BEAM_FUSED=0 runs an iteration as two launches (expand, merge) instead of the fused step
+    static const bool fused_env = [] {
+        const char *e = getenv("VL_BEAM_FUSED");
+        return !(e && e[0] == '0');
+    }();
+    const bool use_fused = fused_env && !use_sort_merge && merge_threads != 64;
+    const bool aligned = (p->dim % 4 == 0) && (((uintptr_t)queries | (uintptr_t)vectors) % 16 == 0);
+    StepArgs step;
+    step.queries = queries; step.vectors = vectors; step.beams = beams; step.n_vectors = p->n_vectors;
+    step.dim = (int)p->dim; step.nchunks = (int)((p->dim + 3) / 4); step.width = (int)p->width;
+    step.memo = l.memo_slots > 0 ? memo : nullptr;
+    step.memo_shift = 32;
+    if (step.memo) {
+        int lg = 0;
+        while ((1 << lg) < l.memo_slots) ++lg;
+        VL_REQUIRE((1 << lg) == l.memo_slots, "memo slots must be a power of two");
+        step.memo_shift = 32 - lg;
+    }
     const int R = (int)p->speculative_readahead;
     const bool prof = g_prof.enabled != 0;
+    step.count_evals = prof ? 1 : 0;
     hipEvent_t ev[3 * 64];
     if (prof) {
         VL_REQUIRE(R <= 64, "profiling supports speculative_readahead up to 64");
@@ -701,12 +839,22 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
         for (int r = 0; r < R; ++r) {
             ++t;
             if (prof) VL_HIP(hipEventRecord(ev[3 * r], st));
+            a.iter = (int)t;
+            if (use_fused) {
+                step.m = a;
+                rc = launch_step_by_dim(step, aligned, merge_threads == 128 ? 128 : 256, smem, st);
+                if (rc < 0) return rc;
+                if (prof) {
+                    VL_HIP(hipEventRecord(ev[3 * r + 1], st));
+                    VL_HIP(hipEventRecord(ev[3 * r + 2], st));
+                }
+                continue;
+            }
             rc = vl_launch_expand(queries, p->n_rows, vectors, p->n_vectors, p->dim, nullptr, v_ids, l.Vt, beams,
                                   p->n_vectors, p->width, l.m, cand_ids, cand_d, ctrl, (int)t, R, (int)l.E, l.VL,
                                   prof ? 1 : 0, memo, l.memo_slots, st);
             if (rc < 0) return rc;
             if (prof) VL_HIP(hipEventRecord(ev[3 * r + 1], st));
-            a.iter = (int)t;
             if (use_sort_merge)
                 hipLaunchKernelGGL(beam_merge_kernel, dim3((unsigned)p->n_rows), dim3(kQueueThreads), smem, st, a);
             else if (merge_threads == 64)

@@ -18,134 +18,9 @@
 // is the same.
 #include "vl_common.h"
 #include "beam_ctrl.h"
+#include "dist_device.h"
 
 namespace {
-
-__device__ __forceinline__ float clamp_distance(float cos_theta) {
-    float r = (1.0f - cos_theta) * 0.5f;  // kernels.py:109
-    if (r < 0.0f) r = 0.0f;               // kernels.py:110-113
-    else if (r > 1.0f) r = 1.0f;
-    return r;
-}
-
-// Per-row cache of distances already evaluated in this search: slot = hash(id),
-// entry = (distance bits << 32) | id, written and read as one 8-byte access.
-__device__ __forceinline__ uint32_t memo_hash(int32_t id, int shift) { return ((uint32_t)id * 2654435761u) >> shift; }
-__device__ __forceinline__ void memo_store(uint64_t *memo_row, int shift, int32_t id, float d) {
-    memo_row[memo_hash(id, shift)] = ((uint64_t)__builtin_bit_cast(uint32_t, d) << 32) | (uint32_t)id;
-}
-
-// One wavefront: lane j holds candidate id `my_id` (valid when `ok`); the
-// distance of candidate lane j to the query goes to out_d[j].
-template <int CPL, int LPR, int U>
-__device__ __forceinline__ void wave_distances(const float *__restrict__ q_row,
-                                               const float *__restrict__ vectors, int dim,
-                                               int nchunks, int32_t my_id, bool ok,
-                                               float *__restrict__ out_d, uint64_t *memo_row,
-                                               int memo_shift) {
-    constexpr int G = kWave / LPR;
-    const int lane = threadIdx.x & (kWave - 1);
-    const int grp = lane / LPR;
-    const int lig = lane % LPR;
-
-    float4 q[CPL];
-    bool cvalid[CPL];
-#pragma unroll
-    for (int i = 0; i < CPL; ++i) {
-        int c = lig + LPR * i;
-        cvalid[i] = c < nchunks;
-        q[i] = cvalid[i] ? reinterpret_cast<const float4 *>(q_row)[c] : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-
-    uint64_t mask = __ballot(ok);
-    while (mask) {
-        int src[U][G];
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-                if (mask) {
-                    src[u][g] = __builtin_ctzll(mask);
-                    mask &= mask - 1;
-                } else {
-                    src[u][g] = -1;
-                }
-            }
-
-        float4 r[U][CPL];
-        int mysrc[U];
-        int32_t ids[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            int s = src[u][0];
-#pragma unroll
-            for (int g = 1; g < G; ++g) s = (grp == g) ? src[u][g] : s;
-            mysrc[u] = s;
-            int32_t id;
-            if constexpr (G == 1) {
-                id = (s >= 0) ? __builtin_amdgcn_readlane(my_id, s) : 0;
-            } else {
-                id = __shfl(my_id, s >= 0 ? s : 0);
-            }
-            ids[u] = id;
-            const float4 *row = reinterpret_cast<const float4 *>(vectors + (int64_t)id * dim);
-#pragma unroll
-            for (int i = 0; i < CPL; ++i) {
-                if (s >= 0 && cvalid[i]) r[u][i] = row[lig + LPR * i];
-                else r[u][i] = make_float4(0.f, 0.f, 0.f, 0.f);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            float acc = 0.0f;
-#pragma unroll
-            for (int i = 0; i < CPL; ++i) {
-                acc = __builtin_fmaf(r[u][i].x, q[i].x, acc);
-                acc = __builtin_fmaf(r[u][i].y, q[i].y, acc);
-                acc = __builtin_fmaf(r[u][i].z, q[i].z, acc);
-                acc = __builtin_fmaf(r[u][i].w, q[i].w, acc);
-            }
-#pragma unroll
-            for (int h = LPR / 2; h >= 1; h >>= 1) acc = acc + __shfl_xor(acc, h);
-            if (lig == 0 && mysrc[u] >= 0) {
-                float d = clamp_distance(acc);
-                out_d[mysrc[u]] = d;
-                if (memo_row) memo_store(memo_row, memo_shift, ids[u], d);
-            }
-        }
-    }
-}
-
-// Any dimension, any alignment: scalar loads, same summation order.
-__device__ __forceinline__ void wave_distances_generic(const float *__restrict__ q_row,
-                                                       const float *__restrict__ vectors, int dim,
-                                                       int nchunks, int32_t my_id, bool ok,
-                                                       float *__restrict__ out_d, uint64_t *memo_row,
-                                                       int memo_shift) {
-    const int lane = threadIdx.x & (kWave - 1);
-    uint64_t mask = __ballot(ok);
-    while (mask) {
-        int s = __builtin_ctzll(mask);
-        mask &= mask - 1;
-        int32_t id = __builtin_amdgcn_readlane(my_id, s);
-        const float *row = vectors + (int64_t)id * dim;
-        float acc = 0.0f;
-        for (int c = lane; c < nchunks; c += kWave) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                int i = 4 * c + j;
-                if (i < dim) acc = __builtin_fmaf(row[i], q_row[i], acc);
-            }
-        }
-#pragma unroll
-        for (int h = kWave / 2; h >= 1; h >>= 1) acc = acc + __shfl_xor(acc, h);
-        if (lane == 0) {
-            float d = clamp_distance(acc);
-            out_d[s] = d;
-            if (memo_row) memo_store(memo_row, memo_shift, id, d);
-        }
-    }
-}
 
 struct ExpandArgs {
     const float *queries;
