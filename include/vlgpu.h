@@ -147,7 +147,16 @@ typedef struct vl_beam_params {
     int64_t exclude_factor;
     int64_t speculative_readahead;
     int64_t excl_cols;            /* columns of the exclusion tensor, 0 if none */
+    int64_t flags;                /* 0 = default; VL_BEAM_* bits select another form of the same loop */
 } vl_beam_params;
+
+/* Forms of one iteration, all with the same result on [:, :queue_length]:
+ * default        one fused launch (expand + merge phases of a row in one workgroup);
+ * TWO_LAUNCHES   expand kernel, then merge kernel;
+ * SORT_MERGE     two launches, the merge step sorts whole queue rows (exact for
+ *                queue rows in any state, not only in Queue.insert order). */
+#define VL_BEAM_TWO_LAUNCHES 1
+#define VL_BEAM_SORT_MERGE 2
 
 int64_t vl_beam_workspace_bytes(const vl_beam_params *p);
 

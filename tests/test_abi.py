@@ -68,7 +68,7 @@ def test_host_side_validation(lib):
     # beam parameters: queue too small for one round of candidates, workspace too small
     p = nv.BeamParams(n_rows=10, dim=8, n_vectors=100, width=8, queue_capacity=20, queue_length=8, beam_size=4,
                       parallel_visit_count=4, visit_queue_factor=3, exclude_factor=5, speculative_readahead=5,
-                      excl_cols=0)
+                      excl_cols=0, flags=0)
     assert lib.vl_beam_workspace_bytes(C.byref(p)) == -1
     p.queue_capacity = 8 + 32
     need = lib.vl_beam_workspace_bytes(C.byref(p))

@@ -330,6 +330,36 @@ def test_closest_vectors_build_step(n, dim, beam, bqf, pv, vqf, ef, ra, fused):
     assert np.array_equal(bits(host(gq.distances)[:, :ql]), bits(oq.distances[:, :ql]))
 
 
+@pytest.mark.parametrize("ra,ef,vqf", [(5, 2, 2), (1, 1, 2), (2, 3, 1), (3, 1, 3)])
+def test_closest_vectors_many_rows_short_visited_list(ra, ef, vqf):
+    """Thousands of rows per launch with a visited list that fills up after a few iterations:
+    the batch-wide state (first free column, changed flags) is read and raised by
+    workgroups that are in different phases of the same launch."""
+    say(f"closest_vectors 30000 rows, readahead={ra} exclude_factor={ef}")
+    from vectorlink_gpu import Queue
+    from vectorlink_gpu.ann import closest_vectors, excluding_self
+
+    rng = np.random.default_rng(77 + ra)
+    n, dim, beam, bqf, pv = 30000, 8, 4, 2, 4
+    v = unit(rng, n, dim)
+    c = cfg(beam_size=beam, beam_queue_factor=bqf, parallel_visit_count=pv, visit_queue_factor=vqf,
+            exclude_factor=ef, speculative_readahead=ra)
+    ql = beam * bqf
+    beams = orc.generate_circulant_beams(n, orc.primes(ql))
+    d = orc.calculate_distances(v, beams)
+    oq = orc.Queue(n, ql, ql + ql * pv)
+    oq.insert(beams, d)
+    t_want = orc.closest_vectors(v, oq, v, beams, c, orc.excluding_self(0, n))
+    gv, gb = dev(v), dev(beams)
+    for attempt in range(3):  # the interleaving of workgroups differs from run to run
+        gq = Queue(n, ql, ql + ql * pv)
+        gq.insert(gb, dev(d))
+        t_got = closest_vectors(gv, gq, gv, gb, c, excluding_self(0, n))
+        assert t_got == t_want
+        assert np.array_equal(host(gq.indices)[:, :ql], oq.indices[:, :ql])
+        assert np.array_equal(bits(host(gq.distances)[:, :ql]), bits(oq.distances[:, :ql]))
+
+
 def test_generate_ann_and_search_against_oracle():
     say("generate_ann + search, n=1500")
     from vectorlink_gpu import ANN

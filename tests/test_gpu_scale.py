@@ -176,3 +176,33 @@ def test_offsets_beyond_2_to_31_elements():
     assert not bool((qi == own).any())
     assert torch.equal(gather_distances(v[s0:e0], v, qi.contiguous()), qd)
     assert bool((qd[:, 0] <= d[s0:e0].min(dim=1).values).all())       # never worse than the seeds
+
+
+def test_three_forms_of_the_loop_agree_at_scale(mix128):
+    """One batch of 10,000 rows at 1M x 128 through the fused step, the two-launch form and
+    the full-sort merge: same iteration count, same queues, bit for bit."""
+    say("fused vs two launches vs sort merge, 10000 rows of 1M x 128")
+    from vectorlink_gpu import synthetic
+    from vectorlink_gpu.ann import BEAM_SORT_MERGE, BEAM_TWO_LAUNCHES, closest_vectors, excluding_self
+    from vectorlink_gpu.kernels import calculate_distances
+    from vectorlink_gpu.queue import Queue
+    from vectorlink_gpu.utils import generate_circulant_beams, primes
+
+    base, q, w = mix128
+    v = base.to(DEV)
+    n = v.shape[0]
+    cfg = dict(orc.DEFAULT_CONFIG)
+    cfg.update(synthetic.ann_kwargs(w))
+    ql = cfg["beam_size"] * cfg["beam_queue_factor"]
+    beams = generate_circulant_beams(n, primes(ql))
+    d = calculate_distances(v, beams)
+    s0, e0 = 500_000, 510_000
+    results = []
+    for flags in (0, BEAM_TWO_LAUNCHES, BEAM_SORT_MERGE, 0):
+        gq = Queue(e0 - s0, ql, ql + ql * 4)
+        gq.insert(beams[s0:e0], d[s0:e0])
+        t = closest_vectors(v[s0:e0], gq, v, beams, cfg, excluding_self(s0, e0), flags=flags)
+        results.append((t, gq.indices[:, :ql].clone(), gq.distances[:, :ql].clone()))
+    for (t, ids, dist) in results[1:]:
+        assert t == results[0][0]
+        assert torch.equal(ids, results[0][1]) and torch.equal(dist, results[0][2])

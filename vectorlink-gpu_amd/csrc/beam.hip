@@ -92,7 +92,7 @@ __global__ __launch_bounds__(kQueueThreads) void beam_init_kernel(BeamCtrl *ctrl
     if (t == 0) {
         ctrl->stop = 0;
         ctrl->reserved = 0;
-        ctrl->first[0] = ctrl->first[1] = 0;
+        ctrl->first[0] = ctrl->first[1] = ctrl->first[2] = 0;
     }
     if (t < 64) {
         ctrl->changed[t] = 0;
@@ -126,14 +126,14 @@ __global__ __launch_bounds__(kQueueThreads) void beam_merge_kernel(MergeArgs a) 
     const int t = a.iter;
     const int64_t row = blockIdx.x;
     int cnt = a.seen_count[row];
-    int *first_next = &c->first[(t + 1) & 1];
-    if (t >= 2 && c->first[(t - 1) & 1] >= a.E) {
+    int *first_next = &c->first[(t + 1) % 3];
+    if (t >= 2 && c->first[(t - 1) % 3] >= a.E) {
         // the visit queue is no longer fed: every candidate of this iteration is
         // empty and no queue changes; keep the running maximum current
         if (threadIdx.x == 0) atomicMax(first_next, cnt);
         return;
     }
-    const int first = c->first[t & 1];
+    const int first = c->first[t % 3];
     const bool seen_full = first >= a.E;  // add_new_to_seen_ returns None now (utils.py:68-69)
     const bool checking = (t % a.readahead) == 0;
 
@@ -365,11 +365,11 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
     const int32_t *ci = a.cand_ids + row * a.m;
     const float *cd = a.cand_d + row * a.m;
     const int nva = a.VL - a.Vt;
-    int *first_next = &c->first[(t + 1) & 1];
+    int *first_next = &c->first[(t + 1) % 3];
 
     const int stop = FUSED ? 0 : c->stop;
-    const int first_prev = FUSED ? 0 : c->first[(t - 1) & 1];
-    const int first = c->first[t & 1];
+    const int first_prev = FUSED ? 0 : c->first[(t - 1) % 3];
+    const int first = c->first[t % 3];
     int cnt = a.seen_count[row];
     const int seen_bound = min(a.E, a.Vt * (t - 1));
     if constexpr (FUSED) {
@@ -603,7 +603,7 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
     const int64_t row = blockIdx.x;
     if (gate == 1) {
         // the visit queue is no longer fed: every candidate of this iteration is empty
-        if (threadIdx.x == 0) raise_running_max(&c->first[(t + 1) & 1], a.seen_count[row], min(a.E, a.Vt * t));
+        if (threadIdx.x == 0) raise_running_max(&c->first[(t + 1) % 3], a.seen_count[row], min(a.E, a.Vt * t));
         return;
     }
     // ---- expand: ann.py:69-73 (pop the visit heads, gather their neighbour lists, distances) ----
@@ -791,10 +791,11 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
     a.Pc = vl_next_pow2(l.m);
     if (a.Pc < 2) a.Pc = 2;
     // VL_BEAM_MERGE=sort selects the full-row-sort form of the merge step (exact for queue rows in any state)
-    static const bool use_sort_merge = [] {
+    static const bool sort_merge_env = [] {
         const char *e = getenv("VL_BEAM_MERGE");
         return e && e[0] == 's';
     }();
+    const bool use_sort_merge = sort_merge_env || (p->flags & VL_BEAM_SORT_MERGE);
     // threads per row of the merge step: small rows are latency bound and do better with
     // more rows in flight per CU (measured: 128 wins at m=256, E=480; 256 wins at m=512, E=960)
     static const int merge_threads_env = [] {
@@ -813,7 +814,7 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
         const char *e = getenv("VL_BEAM_FUSED");
         return !(e && e[0] == '0');
     }();
-    const bool use_fused = fused_env && !use_sort_merge && merge_threads != 64;
+    const bool use_fused = fused_env && !use_sort_merge && merge_threads != 64 && !(p->flags & VL_BEAM_TWO_LAUNCHES);
     const bool aligned = (p->dim % 4 == 0) && (((uintptr_t)queries | (uintptr_t)vectors) % 16 == 0);
     StepArgs step;
     step.queries = queries; step.vectors = vectors; step.beams = beams; step.n_vectors = p->n_vectors;

@@ -2,9 +2,11 @@
 // Batch-wide facts that the reference obtains with host round trips live here
 // so that the per-iteration kernels can be enqueued back to back:
 //   stop        - set once a checking iteration saw no row change (ann.py:90-91)
-//   first[2]    - largest visited-list fill over all rows, double buffered by
-//                 iteration parity; it is the first column that is empty in
-//                 every row (utils.py:63-66) because rows are kept sorted
+//   first[3]    - largest visited-list fill over all rows, one slot per iteration
+//                 modulo 3 (iteration t reads t-1 and t, raises t+1, and rows of
+//                 one launch may be in different phases); it is the first column
+//                 that is empty in every row (utils.py:63-66) because rows are
+//                 kept sorted
 //   changed[64] - ring of "some row changed" flags, one per checking iteration
 #pragma once
 #include "vl_common.h"
@@ -12,7 +14,7 @@
 struct BeamCtrl {
     int stop;
     int reserved;
-    int first[2];
+    int first[3];
     int changed[64];
     unsigned long long evals[64];  // profiling only: candidate rows actually fetched, striped by workgroup
     unsigned long long wanted[64]; // profiling only: candidate distances asked for (fetched or served by the cache)
@@ -33,7 +35,9 @@ __device__ inline int beam_gate(BeamCtrl *c, int t, int R, int E, bool writer) {
         if (writer) c->stop = 1;
         return 2;
     }
-    if (writer && ((t - 1) % R) == 0) c->changed[((t - 1) / R + 1) & 63] = 0;
-    if (t >= 2 && c->first[(t - 1) & 1] >= E) return 1;
+    // the slot of the check after next: this iteration itself may be a checking one (R == 1)
+    // and rows of one launch set their flag while others are still here
+    if (writer && ((t - 1) % R) == 0) c->changed[((t - 1) / R + 2) & 63] = 0;
+    if (t >= 2 && c->first[(t - 1) % 3] >= E) return 1;
     return 0;
 }

@@ -19,7 +19,8 @@ _ptr = C.c_void_p
 class BeamParams(C.Structure):
     _fields_ = [(n, C.c_int64) for n in (
         "n_rows", "dim", "n_vectors", "width", "queue_capacity", "queue_length", "beam_size",
-        "parallel_visit_count", "visit_queue_factor", "exclude_factor", "speculative_readahead", "excl_cols")]
+        "parallel_visit_count", "visit_queue_factor", "exclude_factor", "speculative_readahead", "excl_cols",
+        "flags")]
 
 
 _SIGNATURES = {

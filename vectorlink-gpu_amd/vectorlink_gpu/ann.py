@@ -20,14 +20,18 @@ from .queue import Queue
 from .utils import add_new_to_seen_, generate_circulant_beams, generate_queue_circulants, primes
 
 
+BEAM_TWO_LAUNCHES = 1  # include/vlgpu.h: VL_BEAM_TWO_LAUNCHES
+BEAM_SORT_MERGE = 2    # include/vlgpu.h: VL_BEAM_SORT_MERGE
+
+
 def _beam_params(batch: int, dim: int, n_vectors: int, width: int, queue: Queue, config: Dict,
-                 excl_cols: int) -> nv.BeamParams:
+                 excl_cols: int, flags: int = 0) -> nv.BeamParams:
     return nv.BeamParams(
         n_rows=batch, dim=dim, n_vectors=n_vectors, width=width, queue_capacity=queue.indices.size(1),
         queue_length=queue.length, beam_size=config["beam_size"],
         parallel_visit_count=config["parallel_visit_count"], visit_queue_factor=config["visit_queue_factor"],
         exclude_factor=config["exclude_factor"], speculative_readahead=config["speculative_readahead"],
-        excl_cols=excl_cols)
+        excl_cols=excl_cols, flags=flags)
 
 
 _WORKSPACES: Dict[str, Tensor] = {}
@@ -79,10 +83,11 @@ def closest_vectors_stepwise(query_vecs: Tensor, search_queue: Queue, vectors: T
 
 @log_time
 def closest_vectors(query_vecs: Tensor, search_queue: Queue, vectors: Tensor, beams: Tensor, config: Dict,
-                    exclude: Optional[Tensor] = None) -> int:
+                    exclude: Optional[Tensor] = None, flags: int = 0) -> int:
     """reference ann.py:38-93.  Updates search_queue in place; returns the
     number of iterations run (the reference returns True).  Rows are exact on
-    [:, :search_queue.length]; the slots beyond are unspecified."""
+    [:, :search_queue.length]; the slots beyond are unspecified.  flags picks
+    another form of the same loop (BEAM_TWO_LAUNCHES, BEAM_SORT_MERGE)."""
     assert query_vecs.dtype == torch.float32 and vectors.dtype == torch.float32 and beams.dtype == torch.int32
     nv.require_gpu(query_vecs, vectors, beams, search_queue.indices, exclude)
     query_vecs = query_vecs.contiguous()
@@ -95,7 +100,7 @@ def closest_vectors(query_vecs: Tensor, search_queue: Queue, vectors: Tensor, be
         assert exclude.dtype == torch.int32 and exclude.size(0) == batch
         excl = exclude.contiguous()
     p = _beam_params(batch, dim, vectors.size(0), beams.size(1), search_queue, config,
-                     0 if excl is None else excl.size(1))
+                     0 if excl is None else excl.size(1), flags)
     need = nv.check(nv.lib().vl_beam_workspace_bytes(ctypes.byref(p)))
     ws = _workspace(need, vectors.device)
     iterations = nv.check(nv.lib().vl_closest_vectors(
