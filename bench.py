@@ -28,11 +28,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
-# Bytes moved past L2 per expand launch, from two rocprofv3 --pmc runs over the first 104 build steps
+# Bytes moved past L2 per launch of the beam-search step, from two rocprofv3 --pmc runs over the first 104 build steps
 # (FETCH_SIZE x 2.0 after calibration against a 1 GiB copy, + WRITE_SIZE x 1.0); the same runs' algorithmic
-# bytes per launch are given beside it.  profiles/expand_kernel_mix-1m-768_hbm_traffic.txt holds the runs.
+# bytes per launch are given beside it.  profiles/beam_step_kernel_mix-1m-768_hbm_traffic.txt holds the runs.
 # Workloads without a recorded counter run report null.
-TRAFFIC = {"mix-1m-768": dict(bytes_per_launch=12.36e9, algorithmic_bytes_per_launch_in_that_run=12.03e9,
+TRAFFIC = {"mix-1m-768": dict(bytes_per_launch=12.26e9, algorithmic_bytes_per_launch_in_that_run=11.79e9,
                               scope="first 104 build steps (25,605 launches)")}
 
 
@@ -166,7 +166,7 @@ def main():
     # the same with every distance the reference algorithm evaluates, including those the per-row cache served
     effective = ((prof["wanted"] * bytes_per_eval + q_loads) / (prof["expand_ms"] / 1e3) / 1e9
                  if prof["expand_ms"] > 0 else 0.0)
-    roofline = dict(bound="hbm", kernel="expand_kernel (gathered cosine distances of the beam search)",
+    roofline = dict(bound="hbm", kernel="beam_step_kernel (one beam-search iteration: gathered cosine distances + queue merge per row)",
                     achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
                     traffic=(TRAFFIC.get(args.workload) or {}).get("bytes_per_launch"),
                     traffic_detail=TRAFFIC.get(args.workload),
