@@ -511,3 +511,30 @@ def test_rank_pruned_build():
     real = want != M
     wd = orc.calculate_distances(v, np.where(real, want, 0).astype(np.int32))
     assert np.array_equal(bits(host(ann.distances)[real]), bits(wd[real]))
+
+
+def test_exact_duplicate_rows_tie_break_by_id():
+    """Exact duplicate vectors (as in the 20M x 384 workload's 2 % duplicates) give exactly equal
+    distances; every queue must then order by id, as the oracle does."""
+    say("duplicate rows: ties broken by id")
+    from vectorlink_gpu import ANN
+
+    rng = np.random.default_rng(41)
+    n, dim = 1600, 24
+    v = unit(rng, n, dim)
+    dup = rng.choice(n, 400, replace=False)
+    v[dup] = v[rng.integers(0, n, 400)]            # a quarter of the rows are copies of other rows
+    kw = dict(beam_size=10, beam_queue_factor=2, recall_search_queue_factor=2, batch_size=600, optimization_loops=2)
+    c = cfg(**kw)
+    wb, wd = orc.generate_ann(v, c)
+    ann = ANN(dev(v), **kw)
+    assert np.array_equal(host(ann.beams), wb)
+    assert np.array_equal(bits(host(ann.distances)), bits(wd))
+    ties = (np.diff(wd, axis=1) == 0) & (wb[:, 1:] != M)
+    assert ties.sum() > 100                          # the case is really exercised
+    assert (wb[:, 1:][ties] > wb[:, :-1][ties]).all()
+    qv = v[rng.integers(0, n, 64)]
+    res = ann.search(dev(qv))
+    want = orc.search(v, wb, qv, c)
+    L = want.length
+    assert np.array_equal(host(res.indices)[:, :L], want.indices[:, :L])
