@@ -87,6 +87,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run one plain 1 GiB device copy (a known-size kernel to scale rocprofv3 counters by)")
     ap.add_argument("--cpu-rows", type=int, default=768)
+    ap.add_argument("--prune", choices=["reference", "rank", "none"], default="reference",
+                    help="reference = prune_ between loops as the reference does (default); rank = detour-count "
+                         "cut with reverse edges at the end (an addition); none = no pruning")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -108,7 +111,7 @@ def main():
     n, dim = base.shape
     log(f"[bench] workload {args.workload}: {n} x {dim}, generated in {time.time() - t0:.1f} s")
     kwargs = synthetic.ann_kwargs(w)
-    cfg = dict(prune=True, parallel_visit_count=4, visit_queue_factor=3, exclude_factor=5, optimization_loops=3,
+    cfg = dict(prune={"reference": True, "rank": "rank", "none": False}[args.prune], parallel_visit_count=4, visit_queue_factor=3, exclude_factor=5, optimization_loops=3,
                batch_size=10_000, speculative_readahead=5, **kwargs)
     vectors = base.to(dev)
     qdev = queries.to(dev)
@@ -184,7 +187,7 @@ def main():
         "config": {"workload": args.workload, "n": n, "dim": dim, "degree": cfg["beam_size"],
                    "build_queue": cfg["beam_size"] * cfg["beam_queue_factor"], "batch_size": cfg["batch_size"],
                    "optimization_loops": cfg["optimization_loops"], "parallel_visit_count": 4,
-                   "build_seeding": "circulant (reference)", "search_seeding": "dense, 32768 entry points",
+                   "prune": args.prune, "build_seeding": "circulant (reference)", "search_seeding": "dense, 32768 entry points",
                    "queries": int(queries.shape[0])},
         "partial": not complete, "build_seconds": t_build, "loops": build.stats,
         "roofline": roofline,

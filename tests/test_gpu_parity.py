@@ -298,6 +298,10 @@ BEAM_CASES = [
     (300, 12, 5, 2, 3, 2, 1, 2),   # small visited list: fills up, the visit queue stops being fed
     (200, 10, 2, 2, 4, 1, 2, 3),   # visit queue shorter than the visit count
     (400, 768, 16, 2, 4, 3, 5, 5),
+    (500, 1536, 24, 3, 4, 3, 5, 5),  # the reference's default configuration at its default dimension
+    (900, 384, 48, 2, 4, 3, 5, 5),   # degree 48, queue 96: candidate rows of 384 slots (not a power of two)
+    (700, 20, 6, 2, 1, 3, 5, 5),     # one visit per iteration
+    (700, 20, 3, 2, 9, 4, 2, 4),     # more visits than a power of two
 ]
 
 
