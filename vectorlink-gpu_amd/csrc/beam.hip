@@ -634,7 +634,7 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
             if (lane == 0 && wm) atomicAdd(&c->wanted[blockIdx.x & 63], (unsigned long long)__popcll(wm));
         }
         if (memo_row && ok) {
-            uint64_t e = memo_row[memo_hash(id, s.memo_shift)];
+            uint64_t e = memo_load(memo_row, s.memo_shift, id);
             if ((int32_t)(uint32_t)e == id) {
                 ld[slot] = __builtin_bit_cast(float, (uint32_t)(e >> 32));
                 ok = false;

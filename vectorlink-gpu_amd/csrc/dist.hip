@@ -108,7 +108,7 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs a) {
     if (a.memo) {
         memo_row = a.memo + ((uint64_t)row << (32 - a.memo_shift));
         if (ok) {
-            uint64_t e = memo_row[memo_hash(id, a.memo_shift)];
+            uint64_t e = memo_load(memo_row, a.memo_shift, id);
             if ((int32_t)(uint32_t)e == id) {
                 out_d[lane] = __builtin_bit_cast(float, (uint32_t)(e >> 32));
                 ok = false;

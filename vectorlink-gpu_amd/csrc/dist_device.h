@@ -13,10 +13,17 @@ __device__ __forceinline__ float clamp_distance(float cos_theta) {
 }
 
 // Per-row cache of distances already evaluated in this search: slot = hash(id),
-// entry = (distance bits << 32) | id, written and read as one 8-byte access.
+// entry = (distance bits << 32) | id.  Several wavefronts read and write a row's
+// table concurrently, so an entry is always moved as ONE relaxed 64-bit atomic
+// access: a reader sees a whole entry (old or new), never the id of one and the
+// distance of another.
 __device__ __forceinline__ uint32_t memo_hash(int32_t id, int shift) { return ((uint32_t)id * 2654435761u) >> shift; }
 __device__ __forceinline__ void memo_store(uint64_t *memo_row, int shift, int32_t id, float d) {
-    memo_row[memo_hash(id, shift)] = ((uint64_t)__builtin_bit_cast(uint32_t, d) << 32) | (uint32_t)id;
+    uint64_t e = ((uint64_t)__builtin_bit_cast(uint32_t, d) << 32) | (uint32_t)id;
+    __hip_atomic_store(memo_row + memo_hash(id, shift), e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t memo_load(const uint64_t *memo_row, int shift, int32_t id) {
+    return __hip_atomic_load(memo_row + memo_hash(id, shift), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // One wavefront: lane j holds candidate id `my_id` (valid when `ok`); the
