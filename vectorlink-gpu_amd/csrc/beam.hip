@@ -94,8 +94,8 @@ __global__ __launch_bounds__(kQueueThreads) void beam_init_kernel(BeamCtrl *ctrl
         ctrl->reserved = 0;
         ctrl->first[0] = ctrl->first[1] = ctrl->first[2] = 0;
     }
-    if (t < 64) {
-        ctrl->changed[t] = 0;
+    if (t < 64) ctrl->changed[t] = 0;
+    if (t < kBeamStripes) {
         ctrl->evals[t] = 0;
         ctrl->wanted[t] = 0;
     }
@@ -615,6 +615,7 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
     const int32_t *visit = a.v_ids + row * a.VL;
     const float *q_row = s.queries + row * s.dim;
     uint64_t *memo_row = s.memo ? s.memo + ((uint64_t)row << (32 - s.memo_shift)) : nullptr;
+    int n_wanted = 0, n_fetched = 0;  // profiling counts of this wavefront
     for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
         const int slot = c0 + lane;
         const bool has = slot < a.m;
@@ -629,10 +630,7 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
             li[slot] = ok ? id : VL_MAXINT;
             if (!ok) ld[slot] = VL_MAXFLOAT;
         }
-        if (s.count_evals) {
-            uint64_t wm = __ballot(ok);
-            if (lane == 0 && wm) atomicAdd(&c->wanted[blockIdx.x & 63], (unsigned long long)__popcll(wm));
-        }
+        if (s.count_evals) n_wanted += __popcll(__ballot(ok));
         if (memo_row && ok) {
             uint64_t e = memo_load(memo_row, s.memo_shift, id);
             if ((int32_t)(uint32_t)e == id) {
@@ -640,14 +638,16 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
                 ok = false;
             }
         }
-        if (s.count_evals) {
-            uint64_t okm = __ballot(ok);
-            if (lane == 0 && okm) atomicAdd(&c->evals[blockIdx.x & 63], (unsigned long long)__popcll(okm));
-        }
+        if (s.count_evals) n_fetched += __popcll(__ballot(ok));
         if constexpr (GENERIC)
             wave_distances_generic(q_row, s.vectors, s.dim, s.nchunks, id, ok, ld + c0, memo_row, s.memo_shift);
         else
             wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, id, ok, ld + c0, memo_row, s.memo_shift);
+    }
+    if (s.count_evals && lane == 0) {
+        const int stripe = (int)((blockIdx.x * (THREADS / kWave) + wave) & (kBeamStripes - 1));
+        if (n_wanted) atomicAdd(&c->wanted[stripe], (unsigned long long)n_wanted);
+        if (n_fetched) atomicAdd(&c->evals[stripe], (unsigned long long)n_fetched);
     }
     __syncthreads();
     // ---- merge: ann.py:75-88 ----
@@ -770,7 +770,7 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
 
     {
         int64_t n = p->n_rows * l.VL;
-        if (n < 64) n = 64;
+        if (n < kBeamStripes) n = kBeamStripes;
         if (n < p->n_rows) n = p->n_rows;
         hipLaunchKernelGGL(beam_init_kernel, dim3((unsigned)((n + kQueueThreads - 1) / kQueueThreads)),
                            dim3(kQueueThreads), 0, st, ctrl, p->n_rows, q_ids, q_dists, (int)p->queue_capacity,
@@ -848,10 +848,7 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
                 step.m = a;
                 rc = launch_step_by_dim(step, aligned, merge_threads == 128 ? 128 : 256, smem, st);
                 if (rc < 0) return rc;
-                if (prof) {
-                    VL_HIP(hipEventRecord(ev[3 * r + 1], st));
-                    VL_HIP(hipEventRecord(ev[3 * r + 2], st));
-                }
+                if (prof) VL_HIP(hipEventRecord(ev[3 * r + 1], st));
                 continue;
             }
             rc = vl_launch_expand(queries, p->n_rows, vectors, p->n_vectors, p->dim, nullptr, v_ids, l.Vt, beams,
@@ -878,8 +875,10 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
                 float ms = 0;
                 VL_HIP(hipEventElapsedTime(&ms, ev[3 * r], ev[3 * r + 1]));
                 g_prof.expand_ms += ms;
-                VL_HIP(hipEventElapsedTime(&ms, ev[3 * r + 1], ev[3 * r + 2]));
-                g_prof.merge_ms += ms;
+                if (!use_fused) {
+                    VL_HIP(hipEventElapsedTime(&ms, ev[3 * r + 1], ev[3 * r + 2]));
+                    g_prof.merge_ms += ms;
+                }
             }
             g_prof.expand_launches += R;
             g_prof.merge_launches += R;
@@ -888,13 +887,13 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
         VL_REQUIRE(t < (1ll << 30), "beam search did not terminate");
     }
     if (prof) {
-        unsigned long long ev_counts[64];
+        static thread_local unsigned long long ev_counts[kBeamStripes];
         VL_HIP(hipMemcpyAsync(ev_counts, ctrl->evals, sizeof(ev_counts), hipMemcpyDeviceToHost, st));
         VL_HIP(hipStreamSynchronize(st));
-        for (int i = 0; i < 64; ++i) g_prof.evals += (int64_t)ev_counts[i];
+        for (int i = 0; i < kBeamStripes; ++i) g_prof.evals += (int64_t)ev_counts[i];
         VL_HIP(hipMemcpyAsync(ev_counts, ctrl->wanted, sizeof(ev_counts), hipMemcpyDeviceToHost, st));
         VL_HIP(hipStreamSynchronize(st));
-        for (int i = 0; i < 64; ++i) g_prof.wanted += (int64_t)ev_counts[i];
+        for (int i = 0; i < kBeamStripes; ++i) g_prof.wanted += (int64_t)ev_counts[i];
         g_prof.rows += p->n_rows;
         g_prof.iterations += t;
         for (int i = 0; i < 3 * R; ++i) (void)hipEventDestroy(ev[i]);

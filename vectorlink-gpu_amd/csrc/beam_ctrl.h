@@ -11,13 +11,16 @@
 #pragma once
 #include "vl_common.h"
 
+constexpr int kBeamStripes = 1024;
+
 struct BeamCtrl {
     int stop;
     int reserved;
     int first[3];
     int changed[64];
-    unsigned long long evals[64];  // profiling only: candidate rows actually fetched, striped by workgroup
-    unsigned long long wanted[64]; // profiling only: candidate distances asked for (fetched or served by the cache)
+    // profiling only, striped by workgroup so that the atomic adds do not queue up on one address:
+    unsigned long long evals[kBeamStripes];   // candidate rows actually fetched
+    unsigned long long wanted[kBeamStripes];  // candidate distances asked for (fetched or served by the cache)
 };
 
 // State of iteration t as seen by a kernel launched for it:

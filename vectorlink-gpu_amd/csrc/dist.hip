@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs a) {
     }
     if (a.count_evals) {
         uint64_t wm = __ballot(ok);
-        if (lane == 0 && wm) atomicAdd(&a.ctrl->wanted[blockIdx.x & 63], (unsigned long long)__popcll(wm));
+        if (lane == 0 && wm) atomicAdd(&a.ctrl->wanted[blockIdx.x & (kBeamStripes - 1)], (unsigned long long)__popcll(wm));
     }
     // A distance evaluated earlier in this search for the same (row, id) is
     // reused: the cached bits are the ones this kernel would produce again.
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs a) {
     }
     if (a.count_evals) {
         uint64_t okm = __ballot(ok);
-        if (lane == 0 && okm) atomicAdd(&a.ctrl->evals[blockIdx.x & 63], (unsigned long long)__popcll(okm));
+        if (lane == 0 && okm) atomicAdd(&a.ctrl->evals[blockIdx.x & (kBeamStripes - 1)], (unsigned long long)__popcll(okm));
     }
     const float *q_row = a.queries + row * a.dim;
     if constexpr (GENERIC)
