@@ -206,3 +206,42 @@ def test_three_forms_of_the_loop_agree_at_scale(mix128):
     for (t, ids, dist) in results[1:]:
         assert t == results[0][0]
         assert torch.equal(ids, results[0][1]) and torch.equal(dist, results[0][2])
+
+
+def test_10m_x_1536_scale():
+    """The shape of the largest BASELINE workload (10M x 1536 fp32 = 61 GB resident): the initial
+    distance table, one beam-search batch at each end of the id range and exact kNN."""
+    say("10M x 1536 (61 GB)")
+    free, _ = torch.cuda.mem_get_info()
+    if free < 100 * 2**30:
+        pytest.skip("needs 100 GB of free device memory")
+    from vectorlink_gpu.ann import closest_vectors, excluding_self
+    from vectorlink_gpu.kernels import calculate_distances, gather_distances, knn_exact
+    from vectorlink_gpu.queue import Queue
+    from vectorlink_gpu.utils import generate_circulant_beams, primes
+
+    n, dim, beam = 10_000_000, 1536, 64
+    g = torch.Generator(device=DEV).manual_seed(4)
+    v = torch.empty((n, dim), dtype=torch.float32, device=DEV)
+    for s in range(0, n, 250_000):
+        e = min(n, s + 250_000)
+        v[s:e] = torch.nn.functional.normalize(torch.randn((e - s, dim), generator=g, device=DEV), dim=1)
+    cfg = dict(orc.DEFAULT_CONFIG)
+    cfg.update(beam_size=beam, beam_queue_factor=2)
+    ql = 2 * beam
+    beams = generate_circulant_beams(n, primes(ql))
+    d = calculate_distances(v, beams)
+    rows = torch.tensor([0, 4_999_999, n - 1], device=DEV)
+    ref = ((1 - (v[rows].double().unsqueeze(1) * v[beams[rows].long()].double()).sum(2)) / 2).clamp(0, 1)
+    assert torch.allclose(d[rows].double(), ref, rtol=1e-5, atol=1e-6)
+    for s0 in (0, n - 2000):
+        gq = Queue(2000, ql, ql + ql * 4)
+        gq.insert(beams[s0:s0 + 2000], d[s0:s0 + 2000])
+        t = closest_vectors(v[s0:s0 + 2000], gq, v, beams, cfg, excluding_self(s0, s0 + 2000))
+        qi, qd = gq.indices[:, :ql], gq.distances[:, :ql]
+        assert t % 5 == 0 and bool((qd[:, 1:] >= qd[:, :-1]).all()) and bool((qi != M).all())
+        assert torch.equal(gather_distances(v[s0:s0 + 2000], v, qi.contiguous()), qd)
+        assert bool((qd[:, 0] <= d[s0:s0 + 2000].min(dim=1).values).all())
+    q = v[torch.tensor([7, n // 2, n - 3], device=DEV)].contiguous()
+    ki, kd = knn_exact(q, v, 5)
+    assert ki[:, 0].tolist() == [7, n // 2, n - 3] and float(kd[:, 0].max()) < 1e-6
