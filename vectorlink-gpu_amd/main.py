@@ -1,7 +1,11 @@
-"""Command line driver (reference: main.py): build an index over random unit vectors,
-measure its self-recall and write the configuration and timings as JSON.
+"""Command line driver: build an index over random unit vectors, measure its
+self-recall, print and store the run as JSON under ./log/.
 
     python vectorlink-gpu_amd/main.py -c 100000 -d 768 -n 32 -P
+
+Takes the flags of the reference's main.py (main.py:24-99, same letters and
+defaults; note that -r and -p default to 6 and 3 there, not to the class
+defaults 3 and 4).
 """
 import argparse
 import json
@@ -11,60 +15,48 @@ import time
 
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
+# (short flag, long flag, default, help) for the integer options; -P/--prune is the one switch
+INT_OPTIONS = [
+    ("-c", "--vector-count", 10_000, "number of vectors"),
+    ("-d", "--vector-dimension", 1536, "dimension of vectors"),
+    ("-n", "--beam_size", 24, "beam size (max number of neighbors)"),
+    ("-l", "--optimization_loops", 3, "cagra loops"),
+    ("-x", "--exclude_factor", 5, "factor larger than visit queue for exclusion buffer"),
+    ("-q", "--visit_queue_factor", 3, "factor larger than beam for visit queue"),
+    ("-f", "--beam_queue_factor", 3, "factor larger than beam for initial beams"),
+    ("-b", "--batch_size", 10_000, "how many vectors/beams to run per batch"),
+    ("-r", "--recall_search_queue_factor", 6, "recall search queue factor"),
+    ("-p", "--parallel_visit_count", 3, "parallel visit count"),
+    ("-s", "--speculative_readahead", 5, "how far to try to read-ahead before checking for progress"),
+]
 
-def main(vectors, configuration):
-    """reference main.py:11-21"""
+
+def parse(argv=None) -> dict:
+    parser = argparse.ArgumentParser(description=__doc__.splitlines()[0])
+    for short, long_, default, text in INT_OPTIONS:
+        parser.add_argument(short, long_, type=int, default=default, help=text)
+    parser.add_argument("-P", "--prune", action="store_true", default=False, help="prune beams")
+    return vars(parser.parse_args(argv))
+
+
+def main(vectors, configuration: dict) -> dict:
+    """Build, measure, and return the configuration extended with the results (reference main.py:11-21)."""
     from vectorlink_gpu.ann import ANN
 
-    args = configuration.copy()
-    args.pop("vector_count")
-    args.pop("vector_dimension")
-    ann = ANN(vectors=vectors, **args)
-    log = ann.dump_logs()
-    configuration = dict(configuration)
-    configuration.update(total_time=log["total_time"], recall=log["recall"], gpu_arch=log["gpu_arch"])
-    return configuration
+    build_args = {k: v for k, v in configuration.items() if k not in ("vector_count", "vector_dimension")}
+    ann = ANN(vectors=vectors, **build_args)
+    report = dict(configuration)
+    report.update({k: v for k, v in ann.dump_logs().items() if k in ("total_time", "recall", "gpu_arch")})
+    return report
 
 
 if __name__ == "__main__":
-    parser = argparse.ArgumentParser()  # flags and defaults of the reference's main.py:24-99
-    parser.add_argument("-c", "--vector-count", help="number of vectors", type=int, default=10_000)
-    parser.add_argument("-d", "--vector-dimension", help="dimension of vectors", type=int, default=1536)
-    parser.add_argument("-P", "--prune", help="prune beams", default=False, action="store_true")
-    parser.add_argument("-n", "--beam_size", help="beam size (max number of neighbors)", type=int, default=24)
-    parser.add_argument("-l", "--optimization_loops", help="cagra loops", type=int, default=3)
-    parser.add_argument("-x", "--exclude_factor", help="factor larger than visit queue for exclusion buffer", type=int,
-                        default=5)
-    parser.add_argument("-q", "--visit_queue_factor", help="factor larger than beam for visit queue", type=int, default=3)
-    parser.add_argument("-f", "--beam_queue_factor", help="factor larger than beam for initial beams", type=int,
-                        default=3)
-    parser.add_argument("-b", "--batch_size", help="how many vectors/beams to run per batch", type=int, default=10_000)
-    parser.add_argument("-r", "--recall_search_queue_factor", help="recall search queue factor", type=int, default=6)
-    parser.add_argument("-p", "--parallel_visit_count", help="parallel visit count", type=int, default=3)
-    parser.add_argument("-s", "--speculative_readahead",
-                        help="how far to try to read-ahead before checking for progress", type=int, default=5)
-    args = parser.parse_args()
-
+    options = parse()
     from vectorlink_gpu.utils import generate_random_vectors
 
-    build_params = {
-        "vector_count": args.vector_count,
-        "vector_dimension": args.vector_dimension,
-        "prune": args.prune,
-        "beam_size": args.beam_size,
-        "parallel_visit_count": args.parallel_visit_count,
-        "beam_queue_factor": args.beam_queue_factor,
-        "visit_queue_factor": args.visit_queue_factor,
-        "exclude_factor": args.exclude_factor,
-        "optimization_loops": args.optimization_loops,
-        "batch_size": args.batch_size,
-        "recall_search_queue_factor": args.recall_search_queue_factor,
-        "speculative_readahead": args.speculative_readahead,
-    }
-    vectors = generate_random_vectors(number_of_vectors=args.vector_count, dimensions=args.vector_dimension)
-    configuration = main(vectors, build_params)
-    os.makedirs("./log", exist_ok=True)
-    log_name = f"./log/experiment-{time.time()}.log"
-    with open(log_name, "w") as w:
-        print(configuration)
-        json.dump(configuration, w)
+    data = generate_random_vectors(number_of_vectors=options["vector_count"], dimensions=options["vector_dimension"])
+    outcome = main(data, options)
+    print(outcome)
+    os.makedirs("log", exist_ok=True)
+    with open(os.path.join("log", f"experiment-{time.time()}.log"), "w") as sink:
+        json.dump(outcome, sink)

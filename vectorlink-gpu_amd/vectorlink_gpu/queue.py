@@ -17,10 +17,10 @@ class Queue:
         self.distances = torch.full((num_queues, capacity), MAXFLOAT, dtype=torch.float32, device=device)
 
     def initialize_from_queue(self, queue):
-        """queue.py:30-35"""
-        head_length = min(queue.length, self.length)
-        self.indices.narrow(1, 0, head_length).copy_(queue.indices.narrow(1, 0, head_length))
-        self.distances.narrow(1, 0, head_length).copy_(queue.distances.narrow(1, 0, head_length))
+        """Take over the head of another queue: its first min(length, other.length) slots (reference queue.py:30-35)."""
+        n = min(queue.length, self.length)
+        self.indices[:, :n] = queue.indices[:, :n]
+        self.distances[:, :n] = queue.distances[:, :n]
 
     def insert(
         self,
@@ -53,13 +53,12 @@ class Queue:
         return None
 
     def print(self, tail: Optional[bool] = False):
-        (_bs, dim) = self.size()
-        print(self.indices.narrow(1, 0, self.length))
-        print(self.distances.narrow(1, 0, self.length))
-        if tail:
-            print("----------------")
-            print(self.indices.narrow(1, self.length, dim - self.length))
-            print(self.distances.narrow(1, self.length, dim - self.length))
+        """Dump the first `length` slots, and with tail=True the slots behind them."""
+        for part in ((slice(0, self.length),) + ((slice(self.length, None),) if tail else ())):
+            if part.start:
+                print("-" * 16)
+            print(self.indices[:, part])
+            print(self.distances[:, part])
 
     def pop_n_ids(self, n: int):
         """queue.py:87-95"""
