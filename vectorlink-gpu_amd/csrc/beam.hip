@@ -2,18 +2,21 @@
 // gfx950.
 //
 // The reference runs ~50 torch ops / Numba launches and at least two blocking
-// host round trips per iteration.  Here an iteration is two launches:
-//   expand  (dist.hip)  pop the visit-queue heads, gather their neighbour
-//                       lists, evaluate the candidate distances;
-//   merge   (this file) one workgroup per query row: insert the candidates
-//                       into the search queue (Queue.insert, queue.py:37-61),
-//                       record the visited ids (add_new_to_seen_,
-//                       utils.py:61-82) and refill the visit queue with the
-//                       candidates not yet visited.
-// Batch-wide state (first free visited-list column, "any row changed") lives
-// in a device control block; the host only reads the changed flag every
-// speculative_readahead iterations, the cadence at which the reference tests
-// for progress (ann.py:68,90-91).
+// host round trips per iteration.  Here an iteration has two phases per query
+// row:
+//   expand  pop the visit-queue heads, gather their neighbour lists, evaluate
+//           the candidate distances (dist_device.h);
+//   merge   insert the candidates into the search queue (Queue.insert,
+//           queue.py:37-61), record the visited ids (add_new_to_seen_,
+//           utils.py:61-82) and refill the visit queue with the candidates
+//           not yet visited.
+// By default both phases of a row run in one workgroup of ONE launch
+// (beam_step_kernel); the two-launch form (expand kernel of dist.hip, then a
+// merge kernel) is kept behind a flag.  Batch-wide state (first free
+// visited-list column, "any row changed") lives in a device control block;
+// the host only reads the changed flag every speculative_readahead
+// iterations, the cadence at which the reference tests for progress
+// (ann.py:68,90-91).
 #include "beam_ctrl.h"
 #include "rowsort.h"
 #include "dist_device.h"
