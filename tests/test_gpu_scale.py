@@ -209,7 +209,7 @@ def test_three_forms_of_the_loop_agree_at_scale(mix128):
 
 
 def test_10m_x_1536_scale():
-    """The shape of the largest BASELINE workload (10M x 1536 fp32 = 61 GB resident): the initial
+    """The shape of the largest workload this library is sized for (10M x 1536 fp32 = 61 GB resident): the initial
     distance table, one beam-search batch at each end of the id range and exact kNN."""
     say("10M x 1536 (61 GB)")
     free, _ = torch.cuda.mem_get_info()

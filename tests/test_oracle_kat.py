@@ -31,7 +31,7 @@ def test_primes_table():
     assert list(orc.primes(4)) == [10000349, 10000357, 10000363, 10000379]
 
 
-# ---------------------------------------------------------------- circulants (KAT B.1)
+# ---------------------------------------------------------------- circulants
 def test_circulant_kat():
     p4 = orc.primes(4)
     got = orc.generate_circulant_beams(10, p4)
@@ -55,7 +55,7 @@ def test_circulant_closed_form(n, k):
     assert np.array_equal(q, np.sort(np.arange(17)[:, None] + p[None, :], axis=1) % n)
 
 
-# ---------------------------------------------------------------- distance (KAT B.2)
+# ---------------------------------------------------------------- distance
 def test_distance_special_cases():
     assert orc.distance_from_cos(1.0) == 0.0
     assert orc.distance_from_cos(0.0) == 0.5
@@ -224,7 +224,7 @@ def test_punchout_excluded_rule():
     assert d[0, 1] == F and d[0, 3] == F and d[0, 4] == np.float32(.5)
 
 
-# ---------------------------------------------------------------- Queue (KAT B.3)
+# ---------------------------------------------------------------- Queue
 def test_queue_kat():
     q = orc.Queue(1, 4, 8)
     q.insert(np.array([[5, 3, 5, 9]]), np.array([[.3, .1, .3, .2]], np.float32))
@@ -262,7 +262,7 @@ def test_queue_initialize_from_queue():
     assert b.indices.tolist() == [[2, M, M, M], [4, M, M, M]]
 
 
-# ---------------------------------------------------------------- prune (KAT B.4)
+# ---------------------------------------------------------------- prune
 def test_prune_kat():
     beams = np.array([[1, 2], [2, 0], [1, 0]], np.int32)
     d = np.array([[.1, .3], [.05, .1], [.05, .3]], np.float32)
