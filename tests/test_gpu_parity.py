@@ -542,3 +542,52 @@ def test_exact_duplicate_rows_tie_break_by_id():
     want = orc.search(v, wb, qv, c)
     L = want.length
     assert np.array_equal(host(res.indices)[:, :L], want.indices[:, :L])
+
+
+def test_closest_vectors_seeded_configuration_sweep():
+    """Forty seeded configurations (sizes, dimensions that are not multiples of 4, queue
+    shapes with and without slack, exclusion lists of several columns, search- and
+    build-shaped calls) through the fused loop against the oracle."""
+    from vectorlink_gpu import Queue
+    from vectorlink_gpu.ann import closest_vectors
+
+    master = np.random.default_rng(2025)
+    for case in range(40):
+        n = int(master.integers(40, 1500))
+        dim = int(master.choice([1, 3, 4, 7, 16, 33, 64, 100, 128, 130, 257, 300]))
+        beam = int(master.integers(1, 20))
+        width = int(master.choice([beam, beam * int(master.integers(1, 4))]))   # neighbour table columns
+        pv = int(master.integers(1, 7))
+        vqf = int(master.integers(1, 4))
+        ef = int(master.integers(1, 6))
+        ra = int(master.integers(1, 7))
+        b = int(master.integers(1, min(n, 400)))
+        length = int(master.integers(1, 50))
+        take = min(vqf * beam, pv)
+        cap = length + max(take * width, min(length, n)) + int(master.choice([0, 0, 5, 40]))
+        excl_cols = int(master.choice([0, 1, 3]))
+        say(f"sweep {case}: n={n} dim={dim} beam={beam} width={width} pv={pv} vqf={vqf} ef={ef} ra={ra} rows={b} "
+            f"length={length} cap={cap} excl={excl_cols}")
+        rng = np.random.default_rng(1000 + case)
+        v = unit(rng, n, dim)
+        q = unit(rng, b, dim)
+        c = cfg(beam_size=beam, parallel_visit_count=pv, visit_queue_factor=vqf, exclude_factor=ef,
+                speculative_readahead=ra)
+        table = np.stack([rng.choice(n, width, replace=width > n) for _ in range(n)]).astype(np.int32)
+        table[rng.random((n, width)) < 0.05] = M
+        seeds = np.stack([rng.choice(n, min(length, n), replace=False) for _ in range(b)]).astype(np.int32)
+        sd = orc.gather_distances(q, v, seeds)
+        ex = None
+        if excl_cols:
+            ex = rng.integers(0, n, (b, excl_cols)).astype(np.int32)
+            if excl_cols == 3:
+                ex[rng.random(b) < 0.5, 1] = M          # lists that end early
+        oq = orc.Queue(b, length, cap)
+        oq.insert(seeds, sd)
+        t_want = orc.closest_vectors(q, oq, v, table, c, ex)
+        gq = Queue(b, length, cap)
+        gq.insert(dev(seeds), dev(sd))
+        t_got = closest_vectors(dev(q), gq, dev(v), dev(table), c, None if ex is None else dev(ex))
+        assert t_got == t_want, case
+        assert np.array_equal(host(gq.indices)[:, :length], oq.indices[:, :length]), case
+        assert np.array_equal(bits(host(gq.distances)[:, :length]), bits(oq.distances[:, :length])), case
