@@ -142,11 +142,15 @@ def main():
     want = args.steps if args.steps > 0 else total_steps
     done = 0
     rows_done = 0
+    t_said = t_start
     for (loop, start, end, iters) in build.steps():
         done += 1
         rows_done += end - start
         if done >= want:
             break
+        if time.time() - t_said > 30.0:   # a long build keeps talking
+            t_said = time.time()
+            log(f"[bench] build: step {done} of {min(want, total_steps)}, loop {loop}, {t_said - t_start:.0f} s")
     torch.cuda.synchronize()
     t_build = time.time() - t_start
     prof = profile_read(nv, reset=True, enable=0)

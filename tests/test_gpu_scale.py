@@ -245,3 +245,84 @@ def test_10m_x_1536_scale():
     q = v[torch.tensor([7, n // 2, n - 3], device=DEV)].contiguous()
     ki, kd = knn_exact(q, v, 5)
     assert ki[:, 0].tolist() == [7, n // 2, n - 3] and float(kd[:, 0].max()) < 1e-6
+
+
+def test_tables_with_more_rows_than_one_launch_holds():
+    """17.5M rows: one workgroup per row at 256 threads would need more than 2^32 threads in
+    one launch, which the hardware queue does not take whole. Every whole-table entry point
+    must cover all rows (checked at both ends of the table and across the seams between launches)."""
+    say("17.5M-row tables: gather, sorts, dedup, prune, queue insert")
+    from vectorlink_gpu.kernels import (dedup_tensor_, gather_distances, index_sort_, knn_exact, optimize_graph, prune_,
+                                        queue_sort_)
+    from vectorlink_gpu.queue import Queue
+
+    n, dim, w = 17_500_000, 4, 4
+    assert n * 256 > 2**32
+    g = torch.Generator(device=DEV).manual_seed(11)
+    v = torch.nn.functional.normalize(torch.randn((n, dim), generator=g, device=DEV), dim=1)
+    ids = torch.randint(0, n, (n, w), generator=g, device=DEV).to(torch.int32)
+    # rows looked at closely: both ends and every seam between launches of 2^21 workgroups
+    step = 1 << 21
+    probe = torch.cat([torch.arange(0, 2000), torch.arange(n - 2000, n)]
+                      + [torch.arange(s - 500, s + 500) for s in range(step, n, step)]).to(DEV)
+
+    d = gather_distances(v, v, ids)
+    ref = ((1 - (v[probe].double().unsqueeze(1) * v[ids[probe].long()].double()).sum(2)) / 2).clamp(0, 1)
+    assert torch.allclose(d[probe].double(), ref, rtol=1e-5, atol=1e-6)
+    hv, hi, hd = v.cpu().numpy(), ids.cpu().numpy(), d.cpu().numpy()
+    pr = probe.cpu().numpy()
+    assert np.array_equal(orc.gather_distances(hv[pr], hv, hi[pr]).view(np.uint32), hd[pr].view(np.uint32))
+
+    # prune over the whole table against the oracle, every row
+    say("  prune")
+    gb, gd = prune_(ids.clone(), d.clone())
+    wb, wd = orc.prune_(hi, hd)
+    assert np.array_equal(gb.cpu().numpy(), wb) and np.array_equal(gd.cpu().numpy().view(np.uint32), wd.view(np.uint32))
+    del gb, gd, wb, wd
+
+    # row sorts against torch.sort (random distances: no ties)
+    say("  sorts")
+    si, sd = ids.clone(), d.clone()
+    index_sort_(si, sd)                                   # by (distance, id)
+    order = torch.sort(d, dim=1, stable=True)
+    ties = (order.values[:, 1:] == order.values[:, :-1]).any(dim=1)
+    assert torch.equal(sd, order.values) and torch.equal(si[~ties], torch.gather(ids, 1, order.indices)[~ties])
+    by_id = torch.sort(ids, dim=1).values
+    si = by_id.clone()
+    dedup_tensor_(si)
+    dup = torch.zeros_like(by_id, dtype=torch.bool)
+    dup[:, 1:] = by_id[:, 1:] == by_id[:, :-1]
+    assert torch.equal(si, torch.where(dup, torch.full_like(si, M), by_id))
+    qi, qd = ids.clone(), d.clone()
+    queue_sort_(qi, qd)
+    assert bool((qd[:, 1:] >= qd[:, :-1]).all())
+    assert torch.equal(gather_distances(v, v, torch.where(qi == M, torch.zeros_like(qi), qi))[qi != M], qd[qi != M])
+    del si, sd, qi, qd, order, dup, by_id, ties
+
+    # queue insert into empty queues: the row-wise best `length` distinct candidates in order
+    say("  queue insert")
+    q = Queue(n, 2, 2 + w)
+    q.insert(ids, d)
+    got_i, got_d = q.indices[probe, :2].cpu().numpy(), q.distances[probe, :2].cpu().numpy()
+    oq = orc.Queue(len(pr), 2, 2 + w)
+    oq.insert(hi[pr], hd[pr])
+    assert np.array_equal(got_i, oq.indices[:, :2]) and np.array_equal(got_d.view(np.uint32), oq.distances[:, :2].view(np.uint32))
+    assert bool((q.distances[:, 0] == d.min(dim=1).values).all())
+    del q
+
+    # rank pruning + reverse edges over more rows than one launch
+    say("  optimize_graph, exact kNN")
+    m = 2_300_000
+    table = torch.randint(0, m, (m, 6), generator=g, device=DEV).to(torch.int32)
+    got = optimize_graph(table, 4)
+    assert np.array_equal(got.cpu().numpy(), orc.optimize_graph(table.cpu().numpy(), 4))
+    # exact kNN with more queries than one launch of the merge kernel
+    small = v[:300].contiguous()
+    ki, kd = knn_exact(v[:m].contiguous(), small, 2)
+    tail = slice(m - 3000, m)
+    full = ((1 - v[:m][tail].double() @ small.double().t()) / 2).clamp(0, 1)
+    best = full.topk(2, dim=1, largest=False)
+    assert torch.allclose(kd[tail].double(), best.values, rtol=1e-5, atol=1e-6)
+    clear = (best.values[:, 1] - best.values[:, 0]) > 1e-5
+    assert torch.equal(ki[tail][clear, 0].long(), best.indices[clear, 0])
+    assert bool((ki[:300, 0] == torch.arange(300, device=DEV)).all())

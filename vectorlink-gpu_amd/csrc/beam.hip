@@ -699,6 +699,8 @@ int beam_layout(const vl_beam_params *p, BeamLayout *l) {
                "configuration values must be positive");
     VL_REQUIRE(p->queue_length > 0 && p->queue_length < p->queue_capacity, "queue length must be below its capacity");
     VL_REQUIRE(p->n_vectors < (1ll << 30), "ids must stay below 2^30");
+    VL_REQUIRE(p->n_rows <= kMaxBlocks, "a batch of %lld rows is too large for one call (limit %lld)",
+               (long long)p->n_rows, (long long)kMaxBlocks);
     l->VL = p->visit_queue_factor * p->beam_size;                                      // ann.py:51
     l->Vt = l->VL < p->parallel_visit_count ? l->VL : p->parallel_visit_count;         // queue.py:89
     l->m = l->Vt * p->width;

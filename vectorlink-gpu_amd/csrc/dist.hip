@@ -131,6 +131,24 @@ void launch_fast(const ExpandArgs &a, dim3 grid, hipStream_t st) {
     hipLaunchKernelGGL((expand_kernel<CPL, LPR, U, false>), grid, dim3(256), 0, st, a);
 }
 
+// one launch: c.n_rows * c.parts workgroups, rounded up to whole groups of 8 rows
+void launch_expand_piece(const ExpandArgs &a, bool aligned, hipStream_t st) {
+    const int nchunks = a.nchunks;
+    dim3 grid((unsigned)((a.n_rows + 7) / 8 * 8 * a.parts));
+    if (!aligned || nchunks > 512) {
+        hipLaunchKernelGGL((expand_kernel<1, 64, 1, true>), grid, dim3(256), 0, st, a);
+    } else if (nchunks <= 16) launch_fast<1, 16, 8>(a, grid, st);
+    else if (nchunks <= 32) launch_fast<1, 32, 8>(a, grid, st);
+    else if (nchunks <= 64) launch_fast<1, 64, 8>(a, grid, st);
+    else if (nchunks <= 128) launch_fast<2, 64, 8>(a, grid, st);
+    else if (nchunks <= 192) launch_fast<3, 64, 4>(a, grid, st);
+    else if (nchunks <= 256) launch_fast<4, 64, 4>(a, grid, st);
+    else if (nchunks <= 320) launch_fast<5, 64, 2>(a, grid, st);
+    else if (nchunks <= 384) launch_fast<6, 64, 2>(a, grid, st);
+    else if (nchunks <= 448) launch_fast<7, 64, 2>(a, grid, st);
+    else launch_fast<8, 64, 2>(a, grid, st);
+}
+
 }  // namespace
 
 // Host-side launcher shared by the C entry points and the beam-search loop.
@@ -169,23 +187,23 @@ int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors,
     if (m < a.cw * 4) a.cw = (int)((m + 3) / 4 < 8 ? 8 : (m + 3) / 4);
     if (a.cw > 64) a.cw = 64;
     a.parts = (int)((m + 4 * a.cw - 1) / (4 * a.cw));
-    int64_t row_groups = (n_rows + 7) / 8;
-    int64_t blocks = row_groups * 8 * a.parts;
-    VL_REQUIRE(blocks < (1ll << 31), "launch of %lld workgroups is too large", (long long)blocks);
-    dim3 grid((unsigned)blocks);
-
-    if (!aligned || nchunks > 512) {
-        hipLaunchKernelGGL((expand_kernel<1, 64, 1, true>), grid, dim3(256), 0, st, a);
-    } else if (nchunks <= 16) launch_fast<1, 16, 8>(a, grid, st);
-    else if (nchunks <= 32) launch_fast<1, 32, 8>(a, grid, st);
-    else if (nchunks <= 64) launch_fast<1, 64, 8>(a, grid, st);
-    else if (nchunks <= 128) launch_fast<2, 64, 8>(a, grid, st);
-    else if (nchunks <= 192) launch_fast<3, 64, 4>(a, grid, st);
-    else if (nchunks <= 256) launch_fast<4, 64, 4>(a, grid, st);
-    else if (nchunks <= 320) launch_fast<5, 64, 2>(a, grid, st);
-    else if (nchunks <= 384) launch_fast<6, 64, 2>(a, grid, st);
-    else if (nchunks <= 448) launch_fast<7, 64, 2>(a, grid, st);
-    else launch_fast<8, 64, 2>(a, grid, st);
+    // rows per launch: a multiple of 8 (the XCD mapping) whose workgroups stay below kMaxBlocks
+    const int64_t rows_per_launch = (kMaxBlocks / a.parts) & ~7ll;
+    VL_REQUIRE(rows_per_launch >= 8, "row of %lld candidates is too wide", (long long)m);
+    VL_REQUIRE(ctrl == nullptr || n_rows <= rows_per_launch, "a beam-search batch of %lld rows is too large (limit %lld)",
+               (long long)n_rows, (long long)rows_per_launch);
+    const int64_t memo_row_slots = a.memo ? (1ll << (32 - a.memo_shift)) : 0;
+    for (int64_t r0 = 0; r0 < n_rows; r0 += rows_per_launch) {
+        ExpandArgs c = a;
+        c.n_rows = (n_rows - r0 < rows_per_launch) ? n_rows - r0 : rows_per_launch;
+        c.queries = queries + r0 * dim;
+        if (ids) c.ids = ids + r0 * m;
+        if (visit) c.visit = visit + r0 * visit_stride;
+        if (idx_out) c.idx_out = idx_out + r0 * m;
+        c.dist_out = dist_out + r0 * m;
+        if (c.memo) c.memo = a.memo + r0 * memo_row_slots;
+        launch_expand_piece(c, aligned, st);
+    }
     VL_LAUNCH_CHECK("expand_kernel");
     return VL_OK;
 }

@@ -26,12 +26,13 @@ namespace {
 constexpr int kSlotBits = 12;  // slots per row < 4096
 
 __global__ __launch_bounds__(kQueueThreads) void rank_prune_kernel(const int32_t *__restrict__ beams, int64_t n, int W,
-                                                                  int P, int degree, int32_t *__restrict__ out) {
+                                                                  int P, int degree, int32_t *__restrict__ out,
+                                                                  int64_t row0) {
     extern __shared__ __align__(16) unsigned char smem[];
     uint64_t *keys = reinterpret_cast<uint64_t *>(smem);       // (id, slot) ordered by id, later (count, slot)
     int32_t *ids = reinterpret_cast<int32_t *>(keys + P);       // row x
     int32_t *count = ids + W;
-    const int64_t x = blockIdx.x;
+    const int64_t x = row0 + blockIdx.x;
     for (int j = threadIdx.x; j < W; j += blockDim.x) {
         ids[j] = beams[x * W + j];
         count[j] = 0;
@@ -73,40 +74,41 @@ __global__ __launch_bounds__(kQueueThreads) void rank_prune_kernel(const int32_t
 
 __global__ void rev_keys_kernel(const int32_t *__restrict__ pruned, int64_t n, int degree, int rev_from,
                                 uint64_t *__restrict__ keys, int32_t *__restrict__ vals) {
-    int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= n * rev_from) return;
-    int64_t x = e / rev_from;
-    int k = (int)(e - x * rev_from);
-    int32_t y = pruned[x * degree + k];
-    bool real = y != VL_MAXINT && y >= 0 && y < n;
-    keys[e] = real ? (((uint64_t)(uint32_t)y << kSlotBits) | (uint32_t)k) : ((1ull << (30 + kSlotBits)) | 0ull);
-    vals[e] = (int32_t)x;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n * rev_from;
+         e += (int64_t)gridDim.x * blockDim.x) {
+        int64_t x = e / rev_from;
+        int k = (int)(e - x * rev_from);
+        int32_t y = pruned[x * degree + k];
+        bool real = y != VL_MAXINT && y >= 0 && y < n;
+        keys[e] = real ? (((uint64_t)(uint32_t)y << kSlotBits) | (uint32_t)k) : ((1ull << (30 + kSlotBits)) | 0ull);
+        vals[e] = (int32_t)x;
+    }
 }
 
 // start[y] = first sorted edge whose target is >= y, for y in [0, n]
 __global__ void rev_start_kernel(const uint64_t *__restrict__ keys, int64_t n_edges, int64_t n, int64_t *__restrict__ start) {
-    int64_t y = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (y > n) return;
-    uint64_t want = (uint64_t)y << kSlotBits;
-    int64_t lo = 0, hi = n_edges;
-    while (lo < hi) {
-        int64_t mid = (lo + hi) >> 1;
-        if (keys[mid] < want) lo = mid + 1;
-        else hi = mid;
+    for (int64_t y = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; y <= n; y += (int64_t)gridDim.x * blockDim.x) {
+        uint64_t want = (uint64_t)y << kSlotBits;
+        int64_t lo = 0, hi = n_edges;
+        while (lo < hi) {
+            int64_t mid = (lo + hi) >> 1;
+            if (keys[mid] < want) lo = mid + 1;
+            else hi = mid;
+        }
+        start[y] = lo;
     }
-    start[y] = lo;
 }
 
 __global__ __launch_bounds__(kQueueThreads) void reverse_merge_kernel(const int32_t *__restrict__ pruned, int64_t n,
                                                                      int degree, int keep, int cap,
                                                                      const int32_t *__restrict__ rev_src,
                                                                      const int64_t *__restrict__ start,
-                                                                     int32_t *__restrict__ out) {
+                                                                     int32_t *__restrict__ out, int64_t row0) {
     extern __shared__ __align__(16) unsigned char smem[];
     int32_t *cand = reinterpret_cast<int32_t *>(smem);  // keep | reverse | rest
     uint8_t *ok = reinterpret_cast<uint8_t *>(cand + 2 * degree);
     __shared__ int wave_cnt[kQueueWaves];
-    const int64_t x = blockIdx.x;
+    const int64_t x = row0 + blockIdx.x;
     const int64_t s = start[x];
     const int n_rev = (int)min((int64_t)cap, start[x + 1] - s);
     const int total = keep + n_rev + (degree - keep);
@@ -221,24 +223,30 @@ VL_EXPORT int vl_optimize_graph(const int32_t *beams, int64_t n, int64_t width, 
     int P = vl_next_pow2(width);
     if (P < 2) P = 2;
     size_t smem = (size_t)P * 8 + (size_t)width * 8;
-    hipLaunchKernelGGL(rank_prune_kernel, dim3((unsigned)n), dim3(kQueueThreads), smem, st, beams, n, (int)width, P,
-                       (int)degree, pruned);
+    for (int64_t row0 = 0; row0 < n; row0 += kMaxBlocks) {
+        int64_t rows = n - row0 < kMaxBlocks ? n - row0 : kMaxBlocks;
+        hipLaunchKernelGGL(rank_prune_kernel, dim3((unsigned)rows), dim3(kQueueThreads), smem, st, beams, n, (int)width,
+                           P, (int)degree, pruned, row0);
+    }
     VL_LAUNCH_CHECK("rank_prune_kernel");
 
     if (p.n_edges > 0) {
-        hipLaunchKernelGGL(rev_keys_kernel, dim3((unsigned)((p.n_edges + 255) / 256)), dim3(256), 0, st, pruned, n,
+        hipLaunchKernelGGL(rev_keys_kernel, dim3(vl_grid_for(p.n_edges, 256)), dim3(256), 0, st, pruned, n,
                            (int)degree, p.rev_from, keys_a, vals_a);
         VL_LAUNCH_CHECK("rev_keys_kernel");
         size_t temp = p.temp_bytes;
         VL_HIP(rocprim::radix_sort_pairs(ws + p.off_temp, temp, keys_a, keys_b, vals_a, vals_b, (size_t)p.n_edges, 0,
                                          31 + kSlotBits, st));
     }
-    hipLaunchKernelGGL(rev_start_kernel, dim3((unsigned)((n + 1 + 255) / 256)), dim3(256), 0, st, keys_b, p.n_edges, n,
+    hipLaunchKernelGGL(rev_start_kernel, dim3(vl_grid_for(n + 1, 256)), dim3(256), 0, st, keys_b, p.n_edges, n,
                        start);
     VL_LAUNCH_CHECK("rev_start_kernel");
     size_t smem2 = (size_t)degree * 8 + (size_t)degree * 2 + 16;
-    hipLaunchKernelGGL(reverse_merge_kernel, dim3((unsigned)n), dim3(kQueueThreads), smem2, st, pruned, n, (int)degree,
-                       p.keep, (int)(degree - p.keep), vals_b, start, out);
+    for (int64_t row0 = 0; row0 < n; row0 += kMaxBlocks) {
+        int64_t rows = n - row0 < kMaxBlocks ? n - row0 : kMaxBlocks;
+        hipLaunchKernelGGL(reverse_merge_kernel, dim3((unsigned)rows), dim3(kQueueThreads), smem2, st, pruned, n,
+                           (int)degree, p.keep, (int)(degree - p.keep), vals_b, start, out, row0);
+    }
     VL_LAUNCH_CHECK("reverse_merge_kernel");
     return VL_OK;
 }

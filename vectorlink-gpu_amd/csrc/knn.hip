@@ -137,10 +137,10 @@ __global__ __launch_bounds__(256) void knn_tile_kernel(const float *__restrict__
 }
 
 __global__ __launch_bounds__(kQueueThreads) void knn_merge_kernel(const uint64_t *__restrict__ cand, int n_cand, int P,
-                                                                 int k, int32_t *ids_out, float *d_out) {
+                                                                 int k, int32_t *ids_out, float *d_out, int64_t q0) {
     extern __shared__ __align__(16) unsigned char smem[];
     uint64_t *keys = reinterpret_cast<uint64_t *>(smem);
-    const int64_t q = blockIdx.x;
+    const int64_t q = q0 + blockIdx.x;
     for (int i = threadIdx.x; i < P; i += blockDim.x) keys[i] = i < n_cand ? cand[q * n_cand + i] : kPadKey;
     block_bitonic_sort(keys, P);
     for (int i = threadIdx.x; i < k; i += blockDim.x) {
@@ -203,7 +203,7 @@ VL_EXPORT int vl_knn_exact(const float *queries, int64_t n_queries, const float 
                      (long long)p.bytes);
         return VL_ERR_WORKSPACE;
     }
-    VL_REQUIRE(n_queries < (1ll << 31), "too many queries");
+    VL_REQUIRE(n_queries <= kMaxBlocks * TQ, "too many queries for one call (limit %lld)", (long long)(kMaxBlocks * TQ));
     hipStream_t st = (hipStream_t)stream;
     uint64_t *cand = (uint64_t *)workspace;
     dim3 grid((unsigned)((n_queries + TQ - 1) / TQ), (unsigned)p.n_strips);
@@ -211,8 +211,11 @@ VL_EXPORT int vl_knn_exact(const float *queries, int64_t n_queries, const float 
                        p.strip_len, p.n_strips, cand);
     VL_LAUNCH_CHECK("knn_tile_kernel");
     int P = vl_next_pow2(p.n_cand);
-    hipLaunchKernelGGL(knn_merge_kernel, dim3((unsigned)n_queries), dim3(kQueueThreads), (size_t)P * 8, st, cand,
-                       p.n_cand, P, (int)k, ids_out, dists_out);
+    for (int64_t q0 = 0; q0 < n_queries; q0 += kMaxBlocks) {
+        int64_t rows = n_queries - q0 < kMaxBlocks ? n_queries - q0 : kMaxBlocks;
+        hipLaunchKernelGGL(knn_merge_kernel, dim3((unsigned)rows), dim3(kQueueThreads), (size_t)P * 8, st, cand,
+                           p.n_cand, P, (int)k, ids_out, dists_out, q0);
+    }
     VL_LAUNCH_CHECK("knn_merge_kernel");
     return VL_OK;
 }

@@ -12,13 +12,14 @@
 namespace {
 
 __global__ __launch_bounds__(kQueueThreads) void prune_kernel(const int32_t *beams, const float *dists, int64_t n,
-                                                             int W, int P, int32_t *beams_out, float *dists_out) {
+                                                             int W, int P, int32_t *beams_out, float *dists_out,
+                                                             int64_t row0) {
     extern __shared__ __align__(16) unsigned char smem[];
     uint64_t *keys = reinterpret_cast<uint64_t *>(smem);
     int32_t *ids = reinterpret_cast<int32_t *>(keys + P);
     float *dd = reinterpret_cast<float *>(ids + P);
     int32_t *mark = reinterpret_cast<int32_t *>(dd + P);
-    const int64_t x = blockIdx.x;
+    const int64_t x = row0 + blockIdx.x;
     for (int i = threadIdx.x; i < W; i += blockDim.x) {
         ids[i] = beams[x * W + i];
         dd[i] = dists[x * W + i];
@@ -68,8 +69,11 @@ VL_EXPORT int vl_prune(const int32_t *beams, const float *dists, int64_t n, int6
     int P = vl_next_pow2(width);
     if (P < 2) P = 2;
     size_t smem = (size_t)P * (8 + 4 + 4 + 4);
-    hipLaunchKernelGGL(prune_kernel, dim3((unsigned)n), dim3(kQueueThreads), smem, (hipStream_t)stream, beams, dists,
-                       n, (int)width, P, beams_out, dists_out);
+    for (int64_t row0 = 0; row0 < n; row0 += kMaxBlocks) {
+        int64_t rows = n - row0 < kMaxBlocks ? n - row0 : kMaxBlocks;
+        hipLaunchKernelGGL(prune_kernel, dim3((unsigned)rows), dim3(kQueueThreads), smem, (hipStream_t)stream, beams,
+                           dists, n, (int)width, P, beams_out, dists_out, row0);
+    }
     VL_LAUNCH_CHECK("prune_kernel");
     return VL_OK;
 }

@@ -19,6 +19,7 @@ struct RowArgs {
     int32_t *ids;
     float *dists;
     int64_t rows;
+    int64_t row0;   // first row of this launch
     int cols;       // slots per row (queue capacity)
     int P;          // cols padded to a power of two
     // insert only
@@ -48,7 +49,7 @@ __global__ __launch_bounds__(kQueueThreads) void queue_row_kernel(RowArgs a) {
     __shared__ PlaceScratch ps;
     __shared__ int n_ex_s;
 
-    const int64_t row = blockIdx.x;
+    const int64_t row = a.row0 + blockIdx.x;
     int32_t *ids = a.ids + row * a.cols;
     float *dd = a.dists + row * a.cols;
 
@@ -140,56 +141,59 @@ int launch_row_kernel(RowArgs a, hipStream_t st) {
     size_t smem = (size_t)a.P * 8 + (size_t)a.P * 4 + (size_t)(a.excl_cols > 0 ? a.excl_cols : 0) * 4;
     VL_REQUIRE(smem <= 60 * 1024, "row of %d slots with %d exclusions needs %zu bytes of LDS (limit 61440)", a.cols,
                a.excl_cols, smem);
-    hipLaunchKernelGGL((queue_row_kernel<MODE>), dim3((unsigned)a.rows), dim3(kQueueThreads), smem, st, a);
+    for (a.row0 = 0; a.row0 < a.rows; a.row0 += kMaxBlocks) {
+        int64_t rows = a.rows - a.row0 < kMaxBlocks ? a.rows - a.row0 : kMaxBlocks;
+        hipLaunchKernelGGL((queue_row_kernel<MODE>), dim3((unsigned)rows), dim3(kQueueThreads), smem, st, a);
+    }
     VL_LAUNCH_CHECK("queue_row_kernel");
     return VL_OK;
 }
 
 // ---- elementwise kernels ---------------------------------------------------
 __global__ void mark_kernel(int32_t *ids, int64_t rows, int64_t cols) {
-    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= rows * cols) return;
-    int64_t q = t % cols;
-    if (q + 1 < cols && same_id_ignoring_flag(ids[t], ids[t + 1])) ids[t + 1] |= VL_DUP_FLAG;
+    // slot t only ever writes slot t + 1's flag bit and compares ids without that bit, so slots may go in any order
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < rows * cols; t += (int64_t)gridDim.x * blockDim.x) {
+        int64_t q = t % cols;
+        if (q + 1 < cols && same_id_ignoring_flag(ids[t], ids[t + 1])) ids[t + 1] |= VL_DUP_FLAG;
+    }
 }
 __global__ void punch_kernel(int32_t *ids, float *d, int64_t n) {
-    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= n) return;
-    if (ids[t] & VL_DUP_FLAG) {  // kernels.py:346-349 (VL_MAXINT itself carries the bit)
-        ids[t] = VL_MAXINT;
-        if (d) d[t] = VL_MAXFLOAT;
-    }
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (int64_t)gridDim.x * blockDim.x)
+        if (ids[t] & VL_DUP_FLAG) {  // kernels.py:346-349 (VL_MAXINT itself carries the bit)
+            ids[t] = VL_MAXINT;
+            if (d) d[t] = VL_MAXFLOAT;
+        }
 }
 __global__ void excluded_kernel(int32_t *ids, float *d, int64_t rows, int64_t cols, int64_t is,
                                 int64_t ds, const int32_t *excl, int64_t ec, int64_t es) {
-    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= rows * cols) return;
-    int64_t r = t / cols, q = t % cols;
-    int32_t v = ids[r * is + q];
-    for (int64_t i = 0; i < ec; ++i) {
-        int32_t e = excl[r * es + i];
-        if (e == VL_MAXINT) break;
-        if (e == v) {
-            ids[r * is + q] = VL_MAXINT;
-            d[r * ds + q] = VL_MAXFLOAT;
-            break;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < rows * cols; t += (int64_t)gridDim.x * blockDim.x) {
+        int64_t r = t / cols, q = t % cols;
+        int32_t v = ids[r * is + q];
+        for (int64_t i = 0; i < ec; ++i) {
+            int32_t e = excl[r * es + i];
+            if (e == VL_MAXINT) break;
+            if (e == v) {
+                ids[r * is + q] = VL_MAXINT;
+                d[r * ds + q] = VL_MAXFLOAT;
+                break;
+            }
         }
     }
 }
 __global__ void index_kernel(const uint32_t *a, const int64_t *idx, uint32_t *out, int64_t rows, int64_t cols) {
-    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= rows * cols) return;
-    int64_t r = t / cols;
-    int64_t j = idx[t];
-    out[t] = (j >= 0 && j < cols) ? a[r * cols + j] : 0u;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < rows * cols; t += (int64_t)gridDim.x * blockDim.x) {
+        int64_t r = t / cols;
+        int64_t j = idx[t];
+        out[t] = (j >= 0 && j < cols) ? a[r * cols + j] : 0u;
+    }
 }
 __global__ void pop_kernel(int32_t *ids, float *d, int64_t rows, int64_t cap, int64_t take, int32_t *out) {
-    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= rows * take) return;
-    int64_t r = t / take, q = t % take;
-    out[t] = ids[r * cap + q];
-    ids[r * cap + q] = VL_MAXINT;
-    d[r * cap + q] = VL_MAXFLOAT;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < rows * take; t += (int64_t)gridDim.x * blockDim.x) {
+        int64_t r = t / take, q = t % take;
+        out[t] = ids[r * cap + q];
+        ids[r * cap + q] = VL_MAXINT;
+        d[r * cap + q] = VL_MAXFLOAT;
+    }
 }
 
 // ---- circulant seed rows (utils.py:26-41) ----------------------------------
@@ -223,14 +227,14 @@ __global__ void set_int_kernel(int *p, int v) { *p = v; }
 
 __global__ __launch_bounds__(kQueueThreads) void seen_add_kernel(int32_t *seen, int64_t rows, int cols, int P,
                                                                 const int32_t *visit, int n_visit,
-                                                                const int *first_p) {
+                                                                const int *first_p, int64_t row0) {
     extern __shared__ __align__(16) unsigned char smem[];
     uint64_t *keys = reinterpret_cast<uint64_t *>(smem);
     const int first = *first_p;
     if (first >= cols) return;                                   // utils.py:68-69
     const int n = min(cols - first, n_visit);                    // utils.py:73-75
     if (n == 0) return;
-    const int64_t row = blockIdx.x;
+    const int64_t row = row0 + blockIdx.x;
     int32_t *s = seen + row * cols;
     for (int i = threadIdx.x; i < P; i += blockDim.x) {
         uint64_t k = kPadKey;
@@ -268,7 +272,7 @@ __global__ __launch_bounds__(kQueueThreads) void seen_add_kernel(int32_t *seen, 
     for (int i = run + threadIdx.x; i < cols; i += blockDim.x) s[i] = VL_MAXINT;
 }
 
-inline unsigned blocks_for(int64_t n, int per) { return (unsigned)((n + per - 1) / per); }
+inline unsigned blocks_for(int64_t n, int per) { return vl_grid_for(n, per); }
 
 }  // namespace
 
@@ -407,8 +411,11 @@ VL_EXPORT int vl_seen_add(int32_t *seen, int64_t rows, int64_t cols, const int32
     hipLaunchKernelGGL(seen_first_free_kernel, dim3(blocks_for(cols, 64)), dim3(64), 0, st, seen, rows, cols, first);
     int P = vl_next_pow2(cols);
     if (P < 2) P = 2;
-    hipLaunchKernelGGL(seen_add_kernel, dim3((unsigned)rows), dim3(kQueueThreads), (size_t)P * 8, st, seen, rows,
-                       (int)cols, P, visit, (int)n_visit, first);
+    for (int64_t row0 = 0; row0 < rows; row0 += kMaxBlocks) {
+        int64_t part = rows - row0 < kMaxBlocks ? rows - row0 : kMaxBlocks;
+        hipLaunchKernelGGL(seen_add_kernel, dim3((unsigned)part), dim3(kQueueThreads), (size_t)P * 8, st, seen, rows,
+                           (int)cols, P, visit, (int)n_visit, first, row0);
+    }
     VL_LAUNCH_CHECK("seen_add");
     int h = 0;
     VL_HIP(hipMemcpyAsync(&h, first, sizeof(int), hipMemcpyDeviceToHost, st));

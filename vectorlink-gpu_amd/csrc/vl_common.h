@@ -40,6 +40,18 @@ void vl_set_error(const char *fmt, ...);
         }                                                                    \
     } while (0)
 
+// ---- launch size ----------------------------------------------------------
+// A grid of 2^32 threads or more in x is not launched whole and no error is
+// raised for it, so launchers cut their work into pieces of at most
+// kMaxBlocks workgroups (of up to 1024 threads each) and kernels take the
+// index of their first row as an argument.
+constexpr int64_t kMaxBlocks = 1ll << 21;
+// workgroups for an elementwise kernel that strides over n items by its grid size
+static inline unsigned vl_grid_for(int64_t n, int per_block) {
+    int64_t b = (n + per_block - 1) / per_block;
+    return (unsigned)(b < 1 ? 1 : (b > kMaxBlocks ? kMaxBlocks : b));
+}
+
 // ---- sort keys -------------------------------------------------------------
 // A queue slot is ordered by (distance asc, id asc).  The 64-bit key holds an
 // order-preserving image of the float in the high word and the id in the low

@@ -15,6 +15,11 @@ WORKLOADS: Dict[str, Dict] = {
                        beam_size=32, beam_queue_factor=2, recall_search_queue_factor=2),
     "mix-1m-768": dict(n=1_000_000, dim=768, kind="mixture", centres=4096, sigma=0.15, seed=2, queries=10_000,
                        beam_size=64, beam_queue_factor=2, recall_search_queue_factor=2),
+    # cluster sizes follow rank^-1.1 and 2 % of the rows are exact copies of other rows
+    "zipf-20m-384": dict(n=20_000_000, dim=384, kind="zipf", centres=16_384, sigma=0.15, zipf_s=1.1, duplicates=0.02,
+                         seed=3, queries=50_000, beam_size=48, beam_queue_factor=2, recall_search_queue_factor=2),
+    "mix-10m-1536": dict(n=10_000_000, dim=1536, kind="mixture", centres=8192, sigma=0.2, seed=4, queries=100_000,
+                         beam_size=64, beam_queue_factor=2, recall_search_queue_factor=2),
 }
 
 
@@ -22,10 +27,14 @@ def _normalise_(x: Tensor) -> Tensor:
     return torch.nn.functional.normalize(x, dim=1, out=x)
 
 
-def _mixture(gen: torch.Generator, centres: Tensor, count: int, sigma: float, chunk: int = 100_000) -> Tensor:
+def _mixture(gen: torch.Generator, centres: Tensor, count: int, sigma: float, chunk: int = 100_000,
+             weights: Tensor = None) -> Tensor:
     dim = centres.size(1)
     out = torch.empty((count, dim), dtype=torch.float32)
-    assign = torch.randint(0, centres.size(0), (count,), generator=gen)
+    if weights is None:
+        assign = torch.randint(0, centres.size(0), (count,), generator=gen)
+    else:
+        assign = torch.multinomial(weights, count, replacement=True, generator=gen)
     for s in range(0, count, chunk):
         e = min(s + chunk, count)
         noise = torch.randn((e - s, dim), generator=gen, dtype=torch.float32)
@@ -34,18 +43,30 @@ def _mixture(gen: torch.Generator, centres: Tensor, count: int, sigma: float, ch
     return out
 
 
-def make(name: str, n: int = None, queries: int = None) -> Tuple[Tensor, Tensor, Dict]:
+def make(name: str, n: int = None, queries: int = None, centres: int = None) -> Tuple[Tensor, Tensor, Dict]:
     """Returns (vectors [n, dim], queries [q, dim], parameters) as CPU float32 tensors.
-    n / queries override the workload's sizes (the draw order is fixed: base set first)."""
+    n / queries / centres override the workload's sizes (the draw order is fixed: centres, base
+    set, duplicate rows, queries)."""
     w = dict(WORKLOADS[name])
     if n is not None:
         w["n"] = n
     if queries is not None:
         w["queries"] = queries
+    if centres is not None:
+        w["centres"] = centres
     gen = torch.Generator().manual_seed(w["seed"])
     if w["kind"] == "iid":
         base = _normalise_(torch.randn((w["n"], w["dim"]), generator=gen, dtype=torch.float32))
         q = _normalise_(torch.randn((w["queries"], w["dim"]), generator=gen, dtype=torch.float32))
+    elif w["kind"] == "zipf":
+        centres = torch.randn((w["centres"], w["dim"]), generator=gen, dtype=torch.float32)
+        weights = torch.arange(1, w["centres"] + 1, dtype=torch.float64).pow(-w["zipf_s"])
+        base = _mixture(gen, centres, w["n"], w["sigma"], weights=weights)
+        copies = int(w["n"] * w["duplicates"])
+        dst = torch.randperm(w["n"], generator=gen)[:copies]
+        src = torch.randint(0, w["n"], (copies,), generator=gen)
+        base[dst] = base[src]
+        q = _mixture(gen, centres, w["queries"], w["sigma"], weights=weights)
     else:
         centres = torch.randn((w["centres"], w["dim"]), generator=gen, dtype=torch.float32)
         base = _mixture(gen, centres, w["n"], w["sigma"])
