@@ -87,6 +87,7 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run one plain 1 GiB device copy (a known-size kernel to scale rocprofv3 counters by)")
     ap.add_argument("--cpu-rows", type=int, default=768)
+    ap.add_argument("--loops", type=int, default=3, help="optimisation loops of the build (the reference's default is 3)")
     ap.add_argument("--prune", choices=["reference", "rank", "none"], default="reference",
                     help="reference = prune_ between loops as the reference does (default); rank = detour-count "
                          "cut with reverse edges at the end (an addition); none = no pruning")
@@ -111,7 +112,7 @@ def main():
     n, dim = base.shape
     log(f"[bench] workload {args.workload}: {n} x {dim}, generated in {time.time() - t0:.1f} s")
     kwargs = synthetic.ann_kwargs(w)
-    cfg = dict(prune={"reference": True, "rank": "rank", "none": False}[args.prune], parallel_visit_count=4, visit_queue_factor=3, exclude_factor=5, optimization_loops=3,
+    cfg = dict(prune={"reference": True, "rank": "rank", "none": False}[args.prune], parallel_visit_count=4, visit_queue_factor=3, exclude_factor=5, optimization_loops=args.loops,
                batch_size=10_000, speculative_readahead=5, **kwargs)
     vectors = base.to(dev)
     qdev = queries.to(dev)

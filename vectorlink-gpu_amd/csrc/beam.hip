@@ -763,6 +763,8 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
         return VL_ERR_WORKSPACE;
     }
     VL_REQUIRE(p->n_rows * (l.VL > l.m ? l.VL : l.m) < (1ll << 40), "batch too large");
+    VL_REQUIRE(p->n_rows * (int64_t)l.VL < (1ll << 31), "batch too large: %lld rows with visit queues of %d slots",
+               (long long)p->n_rows, (int)l.VL);
     hipStream_t st = (hipStream_t)stream;
     char *ws = (char *)workspace;
     int32_t *cand_ids = (int32_t *)(ws + l.off_cand_ids);
