@@ -406,7 +406,10 @@ def test_generate_ann_stale_distance_mode():
 
 # ---------------------------------------------------------------- exact kNN tiles
 @pytest.mark.parametrize("n,dim,nq,k", [(5000, 128, 300, 10), (3000, 768, 129, 10), (1000, 20, 7, 16), (700, 36, 260, 1),
-                                        (130, 8, 5, 10), (20000, 64, 64, 10)])
+                                        (130, 8, 5, 10), (20000, 64, 64, 10),
+                                        # odd numbers of 32-float stages, ragged last stages, every list length
+                                        (4000, 96, 200, 4), (2500, 160, 130, 8), (6000, 100, 50, 12), (300, 32, 1, 16),
+                                        (50000, 32, 1000, 10), (90, 4, 3, 2)])
 def test_knn_exact(n, dim, nq, k):
     say(f"knn_exact n={n} dim={dim} nq={nq} k={k}")
     from vectorlink_gpu.kernels import knn_exact

@@ -4,25 +4,37 @@
 // only contraction-shaped step of the path.
 //
 // One workgroup (4 wavefronts, 2 x 2) owns 128 queries and a strip of the
-// vector set; per step it forms the 128 x 128 tile of dot products with
+// vector set; operand tiles go from global memory straight into LDS
+// (global_load_lds, double-buffered: the next stage lands while this one is
+// multiplied); per step it forms the 128 x 128 tile of dot products with
 // v_mfma_f32_32x32x2_f32 (vectors are the M side, queries the N side, so a
 // lane's 16 accumulator values all belong to ONE query) and every lane keeps a
 // private sorted list of the k best (distance, id) keys for each of its two
 // query columns.  The Q x N distance matrix never exists in memory.  A second
 // kernel merges the per-lane lists of a query in LDS.
+#include <type_traits>
+
 #include "rowsort.h"
 
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int KK = 16;        // list length kept per lane and query (k <= KK)
+constexpr int KMAX = 16;      // longest list kept per lane and query
 constexpr int TQ = 128;       // queries per workgroup
 constexpr int TV = 128;       // vectors per step
-constexpr int KT = 32;        // floats of the reduction dimension staged per pass
-constexpr int LDS_STRIDE = KT + 4;
+constexpr int KT = 32;        // floats of the reduction dimension per stage
+constexpr int CH = KT / 4;    // 16-byte chunks per row and stage
+constexpr int TILE = 128 * KT;  // floats of one staged operand tile (16 KB)
 constexpr int LISTS_PER_STRIP = 4;  // two half-waves x two wave rows see the same query
+constexpr int64_t kResidentWorkgroups = 512;  // MI355X: 256 CUs, two workgroups of this kernel resident on each
 
+typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(1))) const void glb_void;
+
+__device__ __align__(16) const float kZeroChunk[4] = {0.f, 0.f, 0.f, 0.f};
+
+template <int KK>
 __device__ __forceinline__ void list_insert(uint64_t (&key)[KK], uint64_t nk) {
 #pragma unroll
     for (int i = KK - 1; i > 0; --i) {
@@ -32,19 +44,87 @@ __device__ __forceinline__ void list_insert(uint64_t (&key)[KK], uint64_t nk) {
     if (nk < key[0]) key[0] = nk;
 }
 
-__global__ __launch_bounds__(256) void knn_tile_kernel(const float *__restrict__ queries, int64_t n_queries,
+// Chunk c (16 bytes) of tile row r lives in slot r * CH + (c ^ swz(r)): sixteen consecutive
+// rows read the same chunk index from sixteen different 16-byte bank groups.
+__device__ __forceinline__ int swz(int r) { return (r >> 1) & (CH - 1); }
+
+// Staging: 128 rows x KT floats of an operand go straight from global memory into LDS (no
+// registers in between).  A wavefront instruction fills 1 KB = 8 tile rows and lane i writes
+// slot i of those rows, so it fetches the chunk that belongs there.  Each lane has four such
+// (row, chunk) duties per operand; their source addresses at k = 0 are kept as pointers.
+// Rows past `last` repeat row `last` (their results are discarded later).
+__device__ __forceinline__ void duty_pointers(const float *__restrict__ src, int64_t first, int64_t last, int dim,
+                                              int wave, int lane, const float *(&p)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = 8 * (4 * wave + i) + (lane >> 3);
+        const int c = (lane & (CH - 1)) ^ swz(r);
+        int64_t row = first + r;
+        row = row < last ? row : last;
+        p[i] = src + row * dim + 4 * c;
+    }
+}
+
+// RAGGED: the last stage reaches past `dim`; chunks out there come from a zero chunk.
+template <bool RAGGED>
+__device__ __forceinline__ void stage_operand(const float *const (&p)[4], int kt, int dim, float *tile, int wave,
+                                              int lane) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float *g = p[i] + kt;
+        if constexpr (RAGGED) {
+            const int r = 8 * (4 * wave + i) + (lane >> 3);
+            const int c = (lane & (CH - 1)) ^ swz(r);
+            if (kt + 4 * c >= dim) g = kZeroChunk;
+        }
+        __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(tile + 8 * (4 * wave + i) * KT), 16, 0, 0);
+    }
+}
+
+// distance above which a value cannot enter a list whose last key is `last`
+__device__ __forceinline__ float list_bound(uint64_t last) { return last == kPadKey ? 2.0f : vl_key_dist(last); }
+
+template <int KK>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void knn_tile_kernel(const float *__restrict__ queries, int64_t n_queries,
                                                       const float *__restrict__ vectors, int64_t n_vectors,
                                                       int dim, int64_t strip_len, int n_strips,
-                                                      uint64_t *__restrict__ cand) {
-    __shared__ __align__(16) float sV[TV * LDS_STRIDE];
-    __shared__ __align__(16) float sQ[TQ * LDS_STRIDE];
+                                                      int n_qblocks, int q_group, uint64_t *__restrict__ cand) {
+    // two buffers per operand as separate arrays: the compiler can then tell that the loads
+    // landing in one buffer do not touch the one being read
+    __shared__ __align__(16) float sV0[TILE];
+    __shared__ __align__(16) float sV1[TILE];
+    __shared__ __align__(16) float sQ0[TILE];
+    __shared__ __align__(16) float sQ1[TILE];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wr = wave >> 1, wc = wave & 1;
-    const int64_t q0 = (int64_t)blockIdx.x * TQ;
-    const int strip = blockIdx.y;
+    // Work items (query block, strip) are ordered so that q_group query blocks go through all
+    // strips together; workgroups are dealt to the 8 XCDs round-robin and XCD x takes the x-th
+    // eighth of that order.  The query rows that are re-read for every vector tile then stay in
+    // the XCD's L2, and each vector strip is streamed by q_group workgroups together.
+    int q_block, strip;
+    {
+        const int64_t total = (int64_t)n_qblocks * n_strips;
+        const int64_t per_xcd = (total + 7) >> 3;
+        const int64_t j = blockIdx.x >> 3;
+        const int64_t t = (int64_t)(blockIdx.x & 7) * per_xcd + j;
+        if (j >= per_xcd || t >= total) return;
+        const int64_t full = (int64_t)(n_qblocks / q_group) * q_group * n_strips;  // items of the complete groups
+        if (t < full) {
+            const int64_t per_group = (int64_t)q_group * n_strips;
+            const int64_t g = t / per_group, w = t - g * per_group;
+            strip = (int)(w / q_group);
+            q_block = (int)(g * q_group + (w - (int64_t)strip * q_group));
+        } else {
+            const int rest = n_qblocks % q_group;
+            const int64_t w = t - full;
+            strip = (int)(w / rest);
+            q_block = (n_qblocks / q_group) * q_group + (int)(w - (int64_t)strip * rest);
+        }
+    }
+    const int64_t q0 = (int64_t)q_block * TQ;
     const int64_t v_begin = strip * strip_len;
     const int64_t v_end = min(n_vectors, v_begin + strip_len);
 
@@ -53,75 +133,130 @@ __global__ __launch_bounds__(256) void knn_tile_kernel(const float *__restrict__
     for (int cb = 0; cb < 2; ++cb)
 #pragma unroll
         for (int i = 0; i < KK; ++i) list[cb][i] = kPadKey;
+    // A value can only matter if it is not above the KK-th best seen so far for its query; the
+    // two half-waves hold lists of the same queries, so each uses the tighter of the two bounds.
+    float bound[2] = {2.0f, 2.0f};
 
     const int half = lane >> 5;   // which k of an MFMA pair this lane feeds
     const int l32 = lane & 31;
 
-    for (int64_t vt = v_begin; vt < v_end; vt += TV) {
-        floatx16 acc[2][2];
+    // Byte offset of this lane's first 16-byte read in a tile for each of its operand rows;
+    // the read of step g is that offset with bits 5..6 flipped by g (the chunk swizzle).
+    int a_off[2], b_off[2];
 #pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-            for (int cb = 0; cb < 2; ++cb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[rb][cb][r] = 0.0f;
+    for (int i = 0; i < 2; ++i) {
+        int ra = 64 * wr + 32 * i + l32, rb = 64 * wc + 32 * i + l32;
+        a_off[i] = ra * (KT * 4) | ((half ^ swz(ra)) << 4);
+        b_off[i] = rb * (KT * 4) | ((half ^ swz(rb)) << 4);
+    }
+    const bool ragged = (dim % KT) != 0;
+    const float *qp[4], *vp[4];
+    duty_pointers(queries, q0, n_queries - 1, dim, wave, lane, qp);
 
-        for (int kt = 0; kt < dim; kt += KT) {
-            // stage 128 x KT of both operands through registers into LDS
-            float4 rv[4], rq[4];
+    floatx16 acc[2][2];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                int f = tid + 256 * i;
-                int row = f >> 3, c4 = f & 7;
-                int k = kt + 4 * c4;
-                int64_t v = vt + row, q = q0 + row;
-                rv[i] = (v < v_end && k < dim) ? *reinterpret_cast<const float4 *>(vectors + v * dim + k)
-                                               : make_float4(0.f, 0.f, 0.f, 0.f);
-                rq[i] = (q < n_queries && k < dim) ? *reinterpret_cast<const float4 *>(queries + q * dim + k)
-                                                   : make_float4(0.f, 0.f, 0.f, 0.f);
-            }
-            __syncthreads();
+    for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                int f = tid + 256 * i;
-                int row = f >> 3, c4 = f & 7;
-                *reinterpret_cast<float4 *>(&sV[row * LDS_STRIDE + 4 * c4]) = rv[i];
-                *reinterpret_cast<float4 *>(&sQ[row * LDS_STRIDE + 4 * c4]) = rq[i];
-            }
-            __syncthreads();
+        for (int cb = 0; cb < 2; ++cb)
 #pragma unroll
-            for (int g = 0; g < KT / 8; ++g) {
-                float4 a[2], b[2];
-#pragma unroll
-                for (int rb = 0; rb < 2; ++rb)
-                    a[rb] = *reinterpret_cast<const float4 *>(&sV[(64 * wr + 32 * rb + l32) * LDS_STRIDE + 8 * g + 4 * half]);
-#pragma unroll
-                for (int cb = 0; cb < 2; ++cb)
-                    b[cb] = *reinterpret_cast<const float4 *>(&sQ[(64 * wc + 32 * cb + l32) * LDS_STRIDE + 8 * g + 4 * half]);
-#pragma unroll
-                for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-                    for (int cb = 0; cb < 2; ++cb) {
-                        acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb].x, b[cb].x, acc[rb][cb], 0, 0, 0);
-                        acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb].y, b[cb].y, acc[rb][cb], 0, 0, 0);
-                        acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb].z, b[cb].z, acc[rb][cb], 0, 0, 0);
-                        acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb].w, b[cb].w, acc[rb][cb], 0, 0, 0);
-                    }
+            for (int r = 0; r < 16; ++r) acc[rb][cb][r] = 0.0f;
+
+    bool more = v_begin < v_end;
+    if (more) {
+        duty_pointers(vectors, v_begin, v_end - 1, dim, wave, lane, vp);
+        if (ragged) {
+            stage_operand<true>(vp, 0, dim, sV0, wave, lane);
+            stage_operand<true>(qp, 0, dim, sQ0, wave, lane);
+        } else {
+            stage_operand<false>(vp, 0, dim, sV0, wave, lane);
+            stage_operand<false>(qp, 0, dim, sQ0, wave, lane);
+        }
+    }
+    int64_t vt = v_begin;   // tile and stage being multiplied
+    int kt = 0;
+    int64_t tile_first = v_begin;   // first vector of the tile whose last stage just ran
+
+    // One stage: wait for its tiles, start the loads of the next stage into the other buffers,
+    // multiply.  Returns true after the last stage of a tile.
+    auto stage = [&](auto which) -> bool {
+        constexpr int B = decltype(which)::value;
+        float *const v_cur = B ? sV1 : sV0, *const q_cur = B ? sQ1 : sQ0;
+        float *const v_nxt = B ? sV0 : sV1, *const q_nxt = B ? sQ0 : sQ1;
+        // this stage's tiles have landed (own loads, then everybody's) and the other
+        // buffers are no longer being read
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __syncthreads();
+        int nkt = kt + KT;
+        int64_t nvt = vt;
+        if (nkt >= dim) {
+            nkt = 0;
+            nvt = vt + TV;
+            if (nvt < v_end) duty_pointers(vectors, nvt, v_end - 1, dim, wave, lane, vp);
+        }
+        const bool has_next = nvt < v_end;
+        if (has_next) {
+            if (ragged) {
+                stage_operand<true>(vp, nkt, dim, v_nxt, wave, lane);
+                stage_operand<true>(qp, nkt, dim, q_nxt, wave, lane);
+            } else {
+                stage_operand<false>(vp, nkt, dim, v_nxt, wave, lane);
+                stage_operand<false>(qp, nkt, dim, q_nxt, wave, lane);
             }
         }
-        // accumulator register r of this lane: vector row 8*(r/4) + 4*half + r%4, query column l32
+        const char *tv = reinterpret_cast<const char *>(v_cur);
+        const char *tq = reinterpret_cast<const char *>(q_cur);
+#pragma unroll
+        for (int g = 0; g < KT / 8; ++g) {
+            float4 a[2], b[2];
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb) a[rb] = *reinterpret_cast<const float4 *>(tv + (a_off[rb] ^ (g << 5)));
+#pragma unroll
+            for (int cb = 0; cb < 2; ++cb) b[cb] = *reinterpret_cast<const float4 *>(tq + (b_off[cb] ^ (g << 5)));
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb) {
+                    acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb].x, b[cb].x, acc[rb][cb], 0, 0, 0);
+                    acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb].y, b[cb].y, acc[rb][cb], 0, 0, 0);
+                    acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb].z, b[cb].z, acc[rb][cb], 0, 0, 0);
+                    acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb].w, b[cb].w, acc[rb][cb], 0, 0, 0);
+                }
+        }
+        const int64_t tile = vt;
+        kt = nkt;
+        vt = nvt;
+        more = has_next;
+        tile_first = tile;
+        return nkt == 0;
+    };
+    int parity = 0;
+    while (more) {
+        // the two stage bodies differ only in which buffers they name
+        const bool tile_done = parity ? stage(std::integral_constant<int, 1>{}) : stage(std::integral_constant<int, 0>{});
+        parity ^= 1;
+        if (!tile_done) continue;
+        // fold the 128 x 128 distances into the lists; accumulator register r of this lane:
+        // vector row 8*(r/4) + 4*half + r%4, query column l32
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
             for (int cb = 0; cb < 2; ++cb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    int64_t v = vt + 64 * wr + 32 * rb + 8 * (r >> 2) + 4 * half + (r & 3);
+                    int64_t v = tile_first + 64 * wr + 32 * rb + 8 * (r >> 2) + 4 * half + (r & 3);
                     float d = (1.0f - acc[rb][cb][r]) * 0.5f;
                     d = d < 0.0f ? 0.0f : (d > 1.0f ? 1.0f : d);
-                    uint64_t nk = vl_make_key((int32_t)v, d);
-                    if (v < v_end && nk < list[cb][KK - 1]) list_insert(list[cb], nk);
+                    if (v < v_end && !(d > bound[cb])) {
+                        uint64_t nk = vl_make_key((int32_t)v, d);
+                        if (nk < list[cb][KK - 1]) list_insert<KK>(list[cb], nk);
+                    }
+                    acc[rb][cb][r] = 0.0f;
                 }
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) {
+            float own = list_bound(list[cb][KK - 1]);
+            bound[cb] = fminf(own, __shfl_xor(own, 32));
+        }
     }
 
     // per query: n_strips * 4 lists of KK keys
@@ -151,7 +286,11 @@ __global__ __launch_bounds__(kQueueThreads) void knn_merge_kernel(const uint64_t
     }
 }
 
+// list lengths the tile kernel is built for: the shortest that holds k is used
+__host__ inline int list_length(int64_t k) { return k <= 1 ? 1 : k <= 4 ? 4 : k <= 8 ? 8 : k <= 10 ? 10 : k <= 12 ? 12 : 16; }
+
 struct KnnPlan {
+    int list_len;
     int n_strips;
     int64_t strip_len;
     int n_cand;
@@ -160,23 +299,33 @@ struct KnnPlan {
 
 int knn_plan(int64_t n_queries, int64_t n_vectors, int64_t dim, int64_t k, KnnPlan *p) {
     VL_REQUIRE(n_queries >= 0 && n_vectors > 0 && dim > 0, "bad sizes");
-    VL_REQUIRE(k >= 1 && k <= KK, "k must be between 1 and %d", KK);
+    VL_REQUIRE(k >= 1 && k <= KMAX, "k must be between 1 and %d", KMAX);
     VL_REQUIRE(dim % 4 == 0, "exact kNN tiles need a dimension that is a multiple of 4");
     VL_REQUIRE(n_vectors < (1ll << 30), "ids must stay below 2^30");
     int64_t q_blocks = (n_queries + TQ - 1) / TQ;
     if (q_blocks < 1) q_blocks = 1;
-    // enough workgroups to fill 256 CUs a few times over, at most 64 strips
-    int64_t strips = (2048 + q_blocks - 1) / q_blocks;
-    int64_t max_by_len = (n_vectors + TV - 1) / TV;
-    if (strips > max_by_len) strips = max_by_len;
-    if (strips > 64) strips = 64;
-    if (strips < 1) strips = 1;
-    int64_t len = (n_vectors + strips - 1) / strips;
-    len = (len + TV - 1) / TV * TV;
-    strips = (n_vectors + len - 1) / len;
+    // The vector set is cut into at most 64 strips of whole tiles; q_blocks * strips workgroups
+    // share kResidentWorkgroups slots (256 CUs x 2 resident workgroups each), so the run lasts
+    // ceil(workgroups / slots) strips' worth of tiles.  Take the strip count with the shortest
+    // run; a strip more costs a sixteenth of a tile (wider merge afterwards).
+    const int64_t tiles = (n_vectors + TV - 1) / TV;
+    int64_t strips = 1, best_cost = -1;
+    for (int64_t s = 1; s <= 64 && s <= tiles; ++s) {
+        int64_t len_t = (tiles + s - 1) / s;
+        int64_t s2 = (tiles + len_t - 1) / len_t;
+        if (s2 != s) continue;
+        int64_t rounds = (q_blocks * s + kResidentWorkgroups - 1) / kResidentWorkgroups;
+        int64_t cost = rounds * len_t * 16 + s;
+        if (best_cost < 0 || cost < best_cost) {
+            best_cost = cost;
+            strips = s;
+        }
+    }
+    int64_t len = (tiles + strips - 1) / strips * TV;
     p->n_strips = (int)strips;
     p->strip_len = len;
-    p->n_cand = (int)(strips * LISTS_PER_STRIP * KK);
+    p->list_len = list_length(k);
+    p->n_cand = (int)(strips * LISTS_PER_STRIP * p->list_len);
     p->bytes = (n_queries > 0 ? n_queries : 1) * (int64_t)p->n_cand * 8;
     return VL_OK;
 }
@@ -206,9 +355,24 @@ VL_EXPORT int vl_knn_exact(const float *queries, int64_t n_queries, const float 
     VL_REQUIRE(n_queries <= kMaxBlocks * TQ, "too many queries for one call (limit %lld)", (long long)(kMaxBlocks * TQ));
     hipStream_t st = (hipStream_t)stream;
     uint64_t *cand = (uint64_t *)workspace;
-    dim3 grid((unsigned)((n_queries + TQ - 1) / TQ), (unsigned)p.n_strips);
-    hipLaunchKernelGGL(knn_tile_kernel, grid, dim3(256), 0, st, queries, n_queries, vectors, n_vectors, (int)dim,
-                       p.strip_len, p.n_strips, cand);
+    const int64_t q_blocks = (n_queries + TQ - 1) / TQ;
+    // query blocks kept together: as many as put about 2 MB of query rows into one L2 (1..8)
+    int64_t q_group = (2ll << 20) / (TQ * dim * 4);
+    q_group = q_group < 1 ? 1 : (q_group > 8 ? 8 : q_group);
+    const int64_t blocks = (q_blocks * p.n_strips + 7) / 8 * 8;
+    VL_REQUIRE(blocks <= kMaxBlocks * 4, "too many tiles for one call");
+#define VL_KNN_LAUNCH(KK)                                                                                      \
+    hipLaunchKernelGGL(knn_tile_kernel<KK>, dim3((unsigned)blocks), dim3(256), 0, st, queries, n_queries, vectors, \
+                       n_vectors, (int)dim, p.strip_len, p.n_strips, (int)q_blocks, (int)q_group, cand)
+    switch (p.list_len) {
+        case 1: VL_KNN_LAUNCH(1); break;
+        case 4: VL_KNN_LAUNCH(4); break;
+        case 8: VL_KNN_LAUNCH(8); break;
+        case 10: VL_KNN_LAUNCH(10); break;
+        case 12: VL_KNN_LAUNCH(12); break;
+        default: VL_KNN_LAUNCH(16); break;
+    }
+#undef VL_KNN_LAUNCH
     VL_LAUNCH_CHECK("knn_tile_kernel");
     int P = vl_next_pow2(p.n_cand);
     for (int64_t q0 = 0; q0 < n_queries; q0 += kMaxBlocks) {
