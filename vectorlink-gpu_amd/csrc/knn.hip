@@ -153,16 +153,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const float *qp[4], *vp[4];
     duty_pointers(queries, q0, n_queries - 1, dim, wave, lane, qp);
 
-    floatx16 acc[2][2];
-#pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-        for (int cb = 0; cb < 2; ++cb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[rb][cb][r] = 0.0f;
-
-    bool more = v_begin < v_end;
-    if (more) {
+    if (v_begin < v_end) {
         duty_pointers(vectors, v_begin, v_end - 1, dim, wave, lane, vp);
         if (ragged) {
             stage_operand<true>(vp, 0, dim, sV0, wave, lane);
@@ -172,13 +163,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             stage_operand<false>(qp, 0, dim, sQ0, wave, lane);
         }
     }
-    int64_t vt = v_begin;   // tile and stage being multiplied
-    int kt = 0;
-    int64_t tile_first = v_begin;   // first vector of the tile whose last stage just ran
 
-    // One stage: wait for its tiles, start the loads of the next stage into the other buffers,
-    // multiply.  Returns true after the last stage of a tile.
-    auto stage = [&](auto which) -> bool {
+    // One stage (tile vt, floats kt .. kt + KT): wait for its operand tiles, start the loads of
+    // the next stage into the other buffers, multiply.  The two instances differ only in which
+    // buffers they name.
+    auto stage = [&](auto which, int64_t vt, int kt, floatx16 (&acc)[2][2]) {
         constexpr int B = decltype(which)::value;
         float *const v_cur = B ? sV1 : sV0, *const q_cur = B ? sQ1 : sQ0;
         float *const v_nxt = B ? sV0 : sV1, *const q_nxt = B ? sQ0 : sQ1;
@@ -187,13 +176,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
         int nkt = kt + KT;
-        int64_t nvt = vt;
+        bool has_next = true;
         if (nkt >= dim) {
+            // the first stage of the next tile goes into the first buffers: possible from here
+            // only if this stage reads the second ones (an odd stage count ends on the first)
             nkt = 0;
-            nvt = vt + TV;
-            if (nvt < v_end) duty_pointers(vectors, nvt, v_end - 1, dim, wave, lane, vp);
+            has_next = B == 1 && vt + TV < v_end;
+            if (has_next) duty_pointers(vectors, vt + TV, v_end - 1, dim, wave, lane, vp);
         }
-        const bool has_next = nvt < v_end;
         if (has_next) {
             if (ragged) {
                 stage_operand<true>(vp, nkt, dim, v_nxt, wave, lane);
@@ -205,52 +195,78 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
         const char *tv = reinterpret_cast<const char *>(v_cur);
         const char *tq = reinterpret_cast<const char *>(q_cur);
+        // operands of step g + 1 are read while the products of step g are formed
+        float4 a[2][2], b[2][2];
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) a[0][rb] = *reinterpret_cast<const float4 *>(tv + a_off[rb]);
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) b[0][cb] = *reinterpret_cast<const float4 *>(tq + b_off[cb]);
 #pragma unroll
         for (int g = 0; g < KT / 8; ++g) {
-            float4 a[2], b[2];
+            const int cur = g & 1, nxt = cur ^ 1;
+            if (g + 1 < KT / 8) {
 #pragma unroll
-            for (int rb = 0; rb < 2; ++rb) a[rb] = *reinterpret_cast<const float4 *>(tv + (a_off[rb] ^ (g << 5)));
+                for (int rb = 0; rb < 2; ++rb)
+                    a[nxt][rb] = *reinterpret_cast<const float4 *>(tv + (a_off[rb] ^ ((g + 1) << 5)));
 #pragma unroll
-            for (int cb = 0; cb < 2; ++cb) b[cb] = *reinterpret_cast<const float4 *>(tq + (b_off[cb] ^ (g << 5)));
+                for (int cb = 0; cb < 2; ++cb)
+                    b[nxt][cb] = *reinterpret_cast<const float4 *>(tq + (b_off[cb] ^ ((g + 1) << 5)));
+            }
+            __builtin_amdgcn_sched_barrier(0);  // keep those reads ahead of this step's products
 #pragma unroll
             for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
                 for (int cb = 0; cb < 2; ++cb) {
-                    acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb].x, b[cb].x, acc[rb][cb], 0, 0, 0);
-                    acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb].y, b[cb].y, acc[rb][cb], 0, 0, 0);
-                    acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb].z, b[cb].z, acc[rb][cb], 0, 0, 0);
-                    acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rb].w, b[cb].w, acc[rb][cb], 0, 0, 0);
+                    acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][rb].x, b[cur][cb].x, acc[rb][cb], 0, 0, 0);
+                    acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][rb].y, b[cur][cb].y, acc[rb][cb], 0, 0, 0);
+                    acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][rb].z, b[cur][cb].z, acc[rb][cb], 0, 0, 0);
+                    acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][rb].w, b[cur][cb].w, acc[rb][cb], 0, 0, 0);
                 }
         }
-        const int64_t tile = vt;
-        kt = nkt;
-        vt = nvt;
-        more = has_next;
-        tile_first = tile;
-        return nkt == 0;
     };
-    int parity = 0;
-    while (more) {
-        // the two stage bodies differ only in which buffers they name
-        const bool tile_done = parity ? stage(std::integral_constant<int, 1>{}) : stage(std::integral_constant<int, 0>{});
-        parity ^= 1;
-        if (!tile_done) continue;
+
+    const bool odd_stages = ((dim + KT - 1) / KT) & 1;
+    for (int64_t vt = v_begin; vt < v_end; vt += TV) {
+        floatx16 acc[2][2];
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+            for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[rb][cb][r] = 0.0f;
+        if (odd_stages && vt != v_begin) {
+            // nobody could prefetch this tile's first stage: load it now, once the first buffers are free
+            __syncthreads();
+            duty_pointers(vectors, vt, v_end - 1, dim, wave, lane, vp);
+            if (ragged) {
+                stage_operand<true>(vp, 0, dim, sV0, wave, lane);
+                stage_operand<true>(qp, 0, dim, sQ0, wave, lane);
+            } else {
+                stage_operand<false>(vp, 0, dim, sV0, wave, lane);
+                stage_operand<false>(qp, 0, dim, sQ0, wave, lane);
+            }
+        }
+        for (int kt = 0; kt < dim; kt += 2 * KT) {
+            stage(std::integral_constant<int, 0>{}, vt, kt, acc);
+            if (kt + KT < dim) stage(std::integral_constant<int, 1>{}, vt, kt + KT, acc);
+        }
         // fold the 128 x 128 distances into the lists; accumulator register r of this lane:
-        // vector row 8*(r/4) + 4*half + r%4, query column l32
+        // vector row 8*(r/4) + 4*half + r%4, query column l32 (ids stay below 2^30)
+        const int vbase = (int)vt + 64 * wr + 4 * half;
+        const int vlimit = (int)v_end;
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
             for (int cb = 0; cb < 2; ++cb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    int64_t v = tile_first + 64 * wr + 32 * rb + 8 * (r >> 2) + 4 * half + (r & 3);
+                    const int v = vbase + (32 * rb + 8 * (r >> 2) + (r & 3));
                     float d = (1.0f - acc[rb][cb][r]) * 0.5f;
                     d = d < 0.0f ? 0.0f : (d > 1.0f ? 1.0f : d);
-                    if (v < v_end && !(d > bound[cb])) {
-                        uint64_t nk = vl_make_key((int32_t)v, d);
+                    if (v < vlimit && !(d > bound[cb])) {
+                        uint64_t nk = vl_make_key(v, d);
                         if (nk < list[cb][KK - 1]) list_insert<KK>(list[cb], nk);
                     }
-                    acc[rb][cb][r] = 0.0f;
                 }
 #pragma unroll
         for (int cb = 0; cb < 2; ++cb) {
