@@ -393,6 +393,28 @@ def test_generate_ann_and_search_against_oracle():
     assert np.array_equal(bits(host(again.distances)), bits(wd))
 
 
+def test_layered_search_against_oracle():
+    say("search_layers / hnsw_calculate_recall")
+    from vectorlink_gpu.ann import ann_recall_test, hnsw_calculate_recall, initial_queue, search_layers
+
+    rng = np.random.default_rng(16)
+    n, dim = 1200, 16
+    v = unit(rng, n, dim)
+    c = cfg(beam_size=8, beam_queue_factor=2, recall_search_queue_factor=2, batch_size=500, optimization_loops=2)
+    fine, _ = orc.generate_ann(v, c)
+    coarse = orc.generate_circulant_beams(n, orc.primes(5))          # a narrower table as the first layer
+    want = orc.initial_queue(v[:300], c)
+    orc.search_layers([coarse, fine], v[:300], want, v, c)
+    got = initial_queue(dev(v[:300]), c)
+    search_layers([dev(coarse), dev(fine)], dev(v[:300]), got, dev(v), c)
+    L = want.length
+    assert np.array_equal(host(got.indices)[:, :L], want.indices[:, :L])
+    assert np.array_equal(bits(host(got.distances)[:, :L]), bits(want.distances[:, :L]))
+    assert hnsw_calculate_recall(dev(v), [dev(coarse), dev(fine)], c, sample=dev(v[:300]), verbose=False) == \
+        orc.hnsw_calculate_recall(v, [coarse, fine], c, sample=v[:300])
+    assert ann_recall_test(dev(v), c) == orc.ann_calculate_recall(v, fine, c, sample=v)
+
+
 def test_generate_ann_stale_distance_mode():
     from vectorlink_gpu.ann import generate_ann
 

@@ -91,6 +91,26 @@ def test_complete_graph_finds_exact_neighbours():
     assert np.allclose(res.distances[:, :k], wd, rtol=1e-5, atol=1e-6)
 
 
+def test_layered_search_ends_on_the_last_layer():
+    # a layered search is one search per neighbour table; with the complete graph as the last
+    # layer every row must find itself whatever the coarse layers did, and one layer alone
+    # equals a plain search
+    rng = np.random.default_rng(15)
+    n, dim = 40, 5
+    v = unit(rng, n, dim)
+    coarse = orc.generate_circulant_beams(n, orc.primes(6))
+    full = np.stack([np.array([j for j in range(n) if j != i]) for i in range(n)]).astype(np.int32)
+    # the queue's spare capacity is sized from the configured beam size: layers may be narrower, not wider
+    c = cfg(beam_size=n - 1, recall_search_queue_factor=1, parallel_visit_count=2, visit_queue_factor=1)
+    assert orc.hnsw_calculate_recall(v, [coarse, full], c) == (n, 1.0)
+    a = orc.initial_queue(v, c)
+    orc.search_layers([coarse], v, a, v, c)
+    b = orc.initial_queue(v, c)
+    orc.closest_vectors(v, b, v, coarse, c, None)
+    assert np.array_equal(a.indices, b.indices) and np.array_equal(a.distances, b.distances)
+    assert orc.hnsw_calculate_recall(v, [coarse], c) == orc.ann_calculate_recall(v, coarse, c)
+
+
 def test_knn_exact_against_numpy():
     rng = np.random.default_rng(13)
     v = unit(rng, 500, 20)

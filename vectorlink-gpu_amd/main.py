@@ -8,6 +8,7 @@ defaults; note that -r and -p default to 6 and 3 there, not to the class
 defaults 3 and 4).
 """
 import argparse
+import itertools
 import json
 import os
 import sys
@@ -48,6 +49,32 @@ def main(vectors, configuration: dict) -> dict:
     report = dict(configuration)
     report.update({k: v for k, v in ann.dump_logs().items() if k in ("total_time", "recall", "gpu_arch")})
     return report
+
+
+def grid_search(vector_count: int = 1_000_000, vector_dimension: int = 1536, log_dir: str = "./grid-log") -> int:
+    """The reference's parameter sweep (ann.py:323-353): one build per combination, one JSON log each.
+    Returns the number of experiments run."""
+    import torch
+
+    from vectorlink_gpu.constants import DEVICE
+    from vectorlink_gpu.utils import generate_random_vectors
+
+    torch.set_default_device(DEVICE)
+    fixed = {"type": "cagra", "vector_count": vector_count, "vector_dimension": vector_dimension, "exclude_factor": 5,
+             "batch_size": 10_000, "beam_queue_factor": 3, "recall_search_queue_factor": 6}
+    swept = {"prune": [True, False], "beam_size": [24, 32, 46], "parallel_visit_count": [1, 4],
+             "optimization_loops": [1, 2], "visit_queue_factor": [3, 4]}
+    vectors = generate_random_vectors(number_of_vectors=vector_count, dimensions=vector_dimension)
+    os.makedirs(log_dir, exist_ok=True)
+    runs = 0
+    for combo in itertools.product(*swept.values()):
+        configuration = dict(fixed, **dict(zip(swept.keys(), combo)))
+        configuration.pop("type")
+        outcome = main(vectors, configuration)
+        with open(os.path.join(log_dir, f"experiment-{time.time()}.log"), "w") as sink:
+            json.dump(outcome, sink)
+        runs += 1
+    return runs
 
 
 if __name__ == "__main__":

@@ -297,6 +297,43 @@ def ann_calculate_recall(vectors: Tensor, beams: Tensor, config: Dict, sample: O
     return (found, found / sample_size)
 
 
+def search_layers(layers, query_vecs: Tensor, search_queue: Queue, vectors: Tensor, config: Dict):
+    """reference ann.py:96-106: one beam search per neighbour table, coarse to fine, each starting
+    from the queue the previous one left.  Every table is [N, width] over the ids of `vectors`;
+    no ids are excluded, because the queries are vectors, not rows of the index."""
+    for layer in layers:
+        closest_vectors(query_vecs, search_queue, vectors, layer.contiguous(), config, None)
+
+
+def hnsw_calculate_recall(vectors: Tensor, hnsw, config: Dict, sample: Optional[Tensor] = None, verbose: bool = True):
+    """reference ann.py:262-284: self-recall@1 of a layered search.  (There the expected ids are
+    built on the CPU and compared with a device tensor; here they live on the device.)"""
+    if sample is None:
+        sample = vectors
+    (sample_size, _) = sample.size()
+    queue = initial_queue(sample.contiguous(), config)
+    search_layers(hnsw, sample, queue, vectors, config)
+    expected = torch.arange(sample_size, device=vectors.device)
+    found = (expected == queue.indices.t()[0]).sum().item()
+    if verbose:
+        print(f"found: {found} / {sample_size}")
+        print(f"recall: {found / sample_size}")
+    return (found, found / sample_size)
+
+
+def print_timestamp(msg):
+    """reference ann.py:297-298"""
+    print(msg)
+
+
+def ann_recall_test(vectors: Tensor, config: Dict):
+    """reference ann.py:287-293: build, then self-recall@1 over the first 10,000 rows"""
+    (beams, _) = generate_ann(vectors, config)
+    print_timestamp("=> ANN generated")
+    prefix = min(vectors.size()[0], 10_000)
+    return ann_calculate_recall(vectors, beams, config, sample=vectors[:prefix])
+
+
 class ANN:
     """reference ann.py:356-489"""
 
