@@ -26,6 +26,36 @@ __device__ __forceinline__ uint64_t memo_load(const uint64_t *memo_row, int shif
     return __hip_atomic_load(memo_row + memo_hash(id, shift), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Folds the partial sums of a group of LPR lanes: lane l += lane l + h for h = LPR/2 ... 1, so the
+// group's first lane ends with the sum in the fixed order.  Steps of 32 and 16 lanes swap register
+// halves / rows (v_permlane32_swap, v_permlane16_swap), steps inside a row of 16 lanes are DPP row
+// shifts: no trip through the LDS crossbar.  Other lanes end with values nobody uses.  The swaps
+// are written as instructions because the compiler's builtin folds its two results into one when
+// both operands hold the same value.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0u, __builtin_bit_cast(unsigned, x), CTRL, 0xf, 0xf, true));
+}
+template <int LPR>
+__device__ __forceinline__ float fold_group(float acc) {
+    static_assert(LPR == 16 || LPR == 32 || LPR == 64, "group sizes of 16, 32 or 64 lanes");
+    if constexpr (LPR == 64) {
+        float lo = acc, hi = acc;  // after the swap: lo = {acc.lo, acc.lo}, hi = {acc.hi, acc.hi}
+        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+        acc = lo + hi;
+    }
+    if constexpr (LPR >= 32) {
+        float even = acc, odd = acc;  // after the swap: even = rows {0, 0, 2, 2}, odd = rows {1, 1, 3, 3}
+        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(even), "+v"(odd));
+        acc = even + odd;
+    }
+    acc = acc + dpp_move<0x108>(acc);  // row_shl:8
+    acc = acc + dpp_move<0x104>(acc);  // row_shl:4
+    acc = acc + dpp_move<0x102>(acc);  // row_shl:2
+    acc = acc + dpp_move<0x101>(acc);  // row_shl:1
+    return acc;
+}
+
 // One wavefront: lane j holds candidate id `my_id` (valid when `ok`); the
 // distance of candidate lane j to the query goes to out_d[j].
 template <int CPL, int LPR, int U>
@@ -96,8 +126,7 @@ __device__ __forceinline__ void wave_distances(const float *__restrict__ q_row,
                 acc = __builtin_fmaf(r[u][i].z, q[i].z, acc);
                 acc = __builtin_fmaf(r[u][i].w, q[i].w, acc);
             }
-#pragma unroll
-            for (int h = LPR / 2; h >= 1; h >>= 1) acc = acc + __shfl_xor(acc, h);
+            acc = fold_group<LPR>(acc);
             if (lig == 0 && mysrc[u] >= 0) {
                 float d = clamp_distance(acc);
                 out_d[mysrc[u]] = d;
@@ -128,8 +157,7 @@ __device__ __forceinline__ void wave_distances_generic(const float *__restrict__
                 if (i < dim) acc = __builtin_fmaf(row[i], q_row[i], acc);
             }
         }
-#pragma unroll
-        for (int h = kWave / 2; h >= 1; h >>= 1) acc = acc + __shfl_xor(acc, h);
+        acc = fold_group<kWave>(acc);
         if (lane == 0) {
             float d = clamp_distance(acc);
             out_d[s] = d;
