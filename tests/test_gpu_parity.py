@@ -616,3 +616,27 @@ def test_closest_vectors_seeded_configuration_sweep():
         assert t_got == t_want, case
         assert np.array_equal(host(gq.indices)[:, :length], oq.indices[:, :length]), case
         assert np.array_equal(bits(host(gq.distances)[:, :length]), bits(oq.distances[:, :length])), case
+
+
+def test_command_line_driver_and_parameter_sweep(tmp_path):
+    say("main.py: parse, main, grid_search")
+    import importlib.util
+    import json
+    import os
+
+    from vectorlink_gpu.utils import generate_random_vectors
+
+    here = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("vl_main", os.path.join(here, "vectorlink-gpu_amd", "main.py"))
+    cli = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(cli)
+    options = cli.parse(["-c", "1500", "-d", "16", "-n", "8", "-b", "500", "-l", "2", "-P"])
+    assert options["vector_count"] == 1500 and options["prune"] is True and options["recall_search_queue_factor"] == 6
+    data = generate_random_vectors(number_of_vectors=1500, dimensions=16)
+    report = cli.main(data, options)
+    assert report["vector_count"] == 1500 and 0.0 <= report["recall"] <= 1.0 and report["total_time"] > 0
+    runs = cli.grid_search(vector_count=600, vector_dimension=8, log_dir=str(tmp_path))
+    logs = sorted(os.listdir(tmp_path))
+    assert runs == 48 and len(logs) == 48
+    one = json.load(open(os.path.join(tmp_path, logs[0])))
+    assert one["vector_count"] == 600 and "recall" in one
