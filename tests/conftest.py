@@ -30,3 +30,17 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(autouse=True)
+def default_device_is_left_alone():
+    """A test (or the code it calls) must not change torch's process-wide default device:
+    tests that follow build CPU tensors with CPU generators and would fail in its wake."""
+    import torch
+
+    before = torch.get_default_device()
+    yield
+    after = torch.get_default_device()
+    if after != before:
+        torch.set_default_device(before)
+        pytest.fail(f"the default torch device was left at {after} (was {before})")

@@ -640,3 +640,23 @@ def test_command_line_driver_and_parameter_sweep(tmp_path):
     assert runs == 48 and len(logs) == 48
     one = json.load(open(os.path.join(tmp_path, logs[0])))
     assert one["vector_count"] == 600 and "recall" in one
+
+
+def test_caller_with_a_cuda_default_device():
+    """The reference's ANN switches torch's default device to the GPU (ann.py:373-375); a caller who
+    has done the same must still get CPU-seeded workloads and a working build."""
+    say("workload generator and build under torch.set_default_device('cuda')")
+    from vectorlink_gpu import ANN, synthetic
+
+    before = torch.get_default_device()
+    try:
+        torch.set_default_device("cuda")
+        base, q, w = synthetic.make("zipf-20m-384", n=3000, queries=16, centres=8)
+        assert base.device.type == "cpu" and q.device.type == "cpu"
+        again, _, _ = synthetic.make("zipf-20m-384", n=3000, queries=16, centres=8)
+        ann = ANN(base, beam_size=8, beam_queue_factor=2, batch_size=1000, optimization_loops=1)
+        res = ann.search(q)
+    finally:
+        torch.set_default_device(before)
+    assert torch.equal(base, again)
+    assert ann.beams.shape == (3000, 8) and res.indices.shape[0] == 16

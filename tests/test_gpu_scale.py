@@ -50,7 +50,7 @@ def test_build_1m_x_128_properties(mix128):
     # the distances are the distances of the ids: recomputed bit for bit, and against float64 on a sample
     again = gather_distances(v, v, ids)
     assert torch.equal(again, d)
-    sample = torch.randint(0, n, (512,), generator=torch.Generator().manual_seed(0))
+    sample = torch.randint(0, n, (512,), generator=torch.Generator(device="cpu").manual_seed(0), device="cpu")
     vs = base[sample].double()
     nb = base[ids[sample.to(DEV)].cpu().long()].double()              # [512, deg, dim]
     ref = ((1 - (vs.unsqueeze(1) * nb).sum(2)) / 2).clamp(0, 1)
@@ -94,7 +94,7 @@ def test_1m_x_768_distances_knn_and_one_batch_on_the_oracle():
     d = calculate_distances(v, beams)
     assert bool(((d >= 0) & (d <= 1)).all())
     # closed form of the circulant table and float64 distances on a sample of rows
-    sample = torch.tensor([0, 1, 777_777, n - 1])
+    sample = torch.tensor([0, 1, 777_777, n - 1], device="cpu")
     p = torch.from_numpy(orc.primes(ql).astype(np.int64))
     want_ids = (sample.unsqueeze(1) + p.unsqueeze(0)) % n
     assert torch.equal(beams[sample.to(DEV)].cpu().long(), want_ids)
@@ -263,8 +263,8 @@ def test_tables_with_more_rows_than_one_launch_holds():
     ids = torch.randint(0, n, (n, w), generator=g, device=DEV).to(torch.int32)
     # rows looked at closely: both ends and every seam between launches of 2^21 workgroups
     step = 1 << 21
-    probe = torch.cat([torch.arange(0, 2000), torch.arange(n - 2000, n)]
-                      + [torch.arange(s - 500, s + 500) for s in range(step, n, step)]).to(DEV)
+    probe = torch.cat([torch.arange(0, 2000, device=DEV), torch.arange(n - 2000, n, device=DEV)]
+                      + [torch.arange(s - 500, s + 500, device=DEV) for s in range(step, n, step)])
 
     d = gather_distances(v, v, ids)
     ref = ((1 - (v[probe].double().unsqueeze(1) * v[ids[probe].long()].double()).sum(2)) / 2).clamp(0, 1)

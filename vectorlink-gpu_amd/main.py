@@ -54,17 +54,16 @@ def main(vectors, configuration: dict) -> dict:
 def grid_search(vector_count: int = 1_000_000, vector_dimension: int = 1536, log_dir: str = "./grid-log") -> int:
     """The reference's parameter sweep (ann.py:323-353): one build per combination, one JSON log each.
     Returns the number of experiments run."""
-    import torch
-
     from vectorlink_gpu.constants import DEVICE
     from vectorlink_gpu.utils import generate_random_vectors
 
-    torch.set_default_device(DEVICE)
+    # the reference switches torch's process-wide default device here (ann.py:373-375); every tensor of
+    # this package names its device instead, so the caller's default stays as it was
     fixed = {"type": "cagra", "vector_count": vector_count, "vector_dimension": vector_dimension, "exclude_factor": 5,
              "batch_size": 10_000, "beam_queue_factor": 3, "recall_search_queue_factor": 6}
     swept = {"prune": [True, False], "beam_size": [24, 32, 46], "parallel_visit_count": [1, 4],
              "optimization_loops": [1, 2], "visit_queue_factor": [3, 4]}
-    vectors = generate_random_vectors(number_of_vectors=vector_count, dimensions=vector_dimension)
+    vectors = generate_random_vectors(number_of_vectors=vector_count, dimensions=vector_dimension, device=DEVICE)
     os.makedirs(log_dir, exist_ok=True)
     runs = 0
     for combo in itertools.product(*swept.values()):

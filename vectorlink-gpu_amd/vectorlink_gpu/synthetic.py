@@ -6,6 +6,8 @@ from typing import Dict, Tuple
 import torch
 from torch import Tensor
 
+CPU = torch.device("cpu")  # every draw names its device: a caller may have changed torch's default
+
 # name -> parameters.  beam_size = graph degree, beam_queue_factor = build queue / degree,
 # recall_search_queue_factor = search queue / degree; the remaining knobs are the class defaults.
 WORKLOADS: Dict[str, Dict] = {
@@ -30,14 +32,14 @@ def _normalise_(x: Tensor) -> Tensor:
 def _mixture(gen: torch.Generator, centres: Tensor, count: int, sigma: float, chunk: int = 100_000,
              weights: Tensor = None) -> Tensor:
     dim = centres.size(1)
-    out = torch.empty((count, dim), dtype=torch.float32)
+    out = torch.empty((count, dim), dtype=torch.float32, device=CPU)
     if weights is None:
-        assign = torch.randint(0, centres.size(0), (count,), generator=gen)
+        assign = torch.randint(0, centres.size(0), (count,), generator=gen, device=CPU)
     else:
         assign = torch.multinomial(weights, count, replacement=True, generator=gen)
     for s in range(0, count, chunk):
         e = min(s + chunk, count)
-        noise = torch.randn((e - s, dim), generator=gen, dtype=torch.float32)
+        noise = torch.randn((e - s, dim), generator=gen, dtype=torch.float32, device=CPU)
         out[s:e] = centres[assign[s:e]] + sigma * noise
         _normalise_(out[s:e])
     return out
@@ -54,21 +56,21 @@ def make(name: str, n: int = None, queries: int = None, centres: int = None) -> 
         w["queries"] = queries
     if centres is not None:
         w["centres"] = centres
-    gen = torch.Generator().manual_seed(w["seed"])
+    gen = torch.Generator(device=CPU).manual_seed(w["seed"])
     if w["kind"] == "iid":
-        base = _normalise_(torch.randn((w["n"], w["dim"]), generator=gen, dtype=torch.float32))
-        q = _normalise_(torch.randn((w["queries"], w["dim"]), generator=gen, dtype=torch.float32))
+        base = _normalise_(torch.randn((w["n"], w["dim"]), generator=gen, dtype=torch.float32, device=CPU))
+        q = _normalise_(torch.randn((w["queries"], w["dim"]), generator=gen, dtype=torch.float32, device=CPU))
     elif w["kind"] == "zipf":
-        centres = torch.randn((w["centres"], w["dim"]), generator=gen, dtype=torch.float32)
-        weights = torch.arange(1, w["centres"] + 1, dtype=torch.float64).pow(-w["zipf_s"])
+        centres = torch.randn((w["centres"], w["dim"]), generator=gen, dtype=torch.float32, device=CPU)
+        weights = torch.arange(1, w["centres"] + 1, dtype=torch.float64, device=CPU).pow(-w["zipf_s"])
         base = _mixture(gen, centres, w["n"], w["sigma"], weights=weights)
         copies = int(w["n"] * w["duplicates"])
-        dst = torch.randperm(w["n"], generator=gen)[:copies]
-        src = torch.randint(0, w["n"], (copies,), generator=gen)
+        dst = torch.randperm(w["n"], generator=gen, device=CPU)[:copies]
+        src = torch.randint(0, w["n"], (copies,), generator=gen, device=CPU)
         base[dst] = base[src]
         q = _mixture(gen, centres, w["queries"], w["sigma"], weights=weights)
     else:
-        centres = torch.randn((w["centres"], w["dim"]), generator=gen, dtype=torch.float32)
+        centres = torch.randn((w["centres"], w["dim"]), generator=gen, dtype=torch.float32, device=CPU)
         base = _mixture(gen, centres, w["n"], w["sigma"])
         q = _mixture(gen, centres, w["queries"], w["sigma"])
     return base, q, w
