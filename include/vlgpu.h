@@ -20,6 +20,12 @@
  *    the call returns without synchronising unless stated otherwise;
  *  - the library allocates no device memory: scratch comes from the caller
  *    as a workspace whose size the matching *_workspace_bytes call reports;
+ *  - threads: every entry point may be called from several host threads at
+ *    once (the reference is driven from one thread).  The library's only
+ *    shared state is the profiling sums of vl_beam_profile (mutex) and the
+ *    thread-local error text.  A workspace belongs to ONE call at a time: the
+ *    beam-search loop keeps its control block, visit queues and visited lists
+ *    in it, so two vl_closest_vectors calls in flight need two workspaces;
  *  - return value 0 is success; a negative value is an error whose text
  *    vl_last_error() returns (thread local).  Shapes are validated on the
  *    host before anything is launched.
@@ -41,6 +47,7 @@ extern "C" {
 #define VL_ERR_ARG (-1)      /* bad shape / null pointer / unsupported size */
 #define VL_ERR_HIP (-2)      /* a HIP runtime call failed */
 #define VL_ERR_WORKSPACE (-3) /* workspace too small */
+#define VL_ERR_STATE (-4)     /* device-side loop state is inconsistent (a workspace used by two calls at once) */
 
 const char *vl_last_error(void);
 int vl_version(void);
@@ -157,6 +164,16 @@ typedef struct vl_beam_params {
  *                queue rows in any state, not only in Queue.insert order). */
 #define VL_BEAM_TWO_LAUNCHES 1
 #define VL_BEAM_SORT_MERGE 2
+/* A different loop, not the reference's: PER_QUERY_STOP ends every row on its
+ * own.  The reference tests for progress over the whole batch (ann.py:90-91),
+ * so every row keeps expanding until the slowest one is quiet.  With this bit a
+ * row stops expanding once the best node it has not visited yet is farther
+ * than the last slot of its search queue (or nothing is left to visit), later
+ * iterations skip it, and the loop ends at the first progress check that finds
+ * every row stopped.  Results differ from the reference's loop (fewer
+ * expansions per row); they are defined by, and tested against, the CPU model
+ * closest_vectors_per_query of the test oracle.  Fused step only. */
+#define VL_BEAM_PER_QUERY_STOP 4
 
 int64_t vl_beam_workspace_bytes(const vl_beam_params *p);
 
@@ -180,7 +197,8 @@ int64_t vl_closest_vectors(const vl_beam_params *p,
  * may be NULL) receives the sums since the last reset: expand ms, merge ms,
  * expand launches, merge launches, candidate rows fetched, query rows,
  * iterations, candidate distances asked for (fetched + served by the per-row
- * cache of already evaluated pairs).  Not thread safe. */
+ * cache of already evaluated pairs).  The sums are kept under a mutex, so
+ * profiled calls from several host threads add up without tearing. */
 int vl_beam_profile(int enable, int reset, double *out);
 
 /* ---- pruning (kernels.py:441-468 prune_) ------------------------------ */

@@ -47,6 +47,7 @@ def test_sentinels_match_reference_constants():
     text = open(HEADER).read()
     assert f"#define VL_MAXINT {MAXINT}" in text
     assert "#define VL_MAXFLOAT 3.4028e37f" in text and MAXFLOAT == 3.4028e37
+    assert "#define VL_ERR_STATE (-4)" in text
     assert PRIMES_HOST.numel() == 965 and int(PRIMES_HOST[0]) == 10000349 and int(PRIMES_HOST[964]) == 1999
 
 

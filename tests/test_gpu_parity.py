@@ -660,3 +660,141 @@ def test_caller_with_a_cuda_default_device():
         torch.set_default_device(before)
     assert torch.equal(base, again)
     assert ann.beams.shape == (3000, 8) and res.indices.shape[0] == 16
+
+
+def test_two_host_threads_on_two_streams():
+    """Two beam searches in flight at once, one host thread and one stream each: each call owns the
+    scratch memory of its (device, stream), so both must equal the oracle, as must two threads that
+    share the default stream (serialised by the workspace lock)."""
+    say("closest_vectors from two host threads")
+    import threading
+
+    from vectorlink_gpu import Queue
+    from vectorlink_gpu.ann import closest_vectors, excluding_self
+
+    rng = np.random.default_rng(4242)
+    n, dim, beam, bqf, pv = 6000, 32, 8, 2, 4
+    v = unit(rng, n, dim)
+    c = cfg(beam_size=beam, beam_queue_factor=bqf, parallel_visit_count=pv)
+    ql = beam * bqf
+    beams = orc.generate_circulant_beams(n, orc.primes(ql))
+    d = orc.calculate_distances(v, beams)
+    parts = [(0, 2500), (2500, 6000)]
+    want = []
+    for (lo, hi) in parts:
+        oq = orc.Queue(hi - lo, ql, ql + ql * pv)
+        oq.insert(beams[lo:hi], d[lo:hi])
+        t = orc.closest_vectors(v[lo:hi], oq, v, beams, c, orc.excluding_self(lo, hi))
+        want.append((t, oq))
+    gv, gb, gd = dev(v), dev(beams), dev(d)
+    torch.cuda.synchronize()
+
+    for own_stream in (True, False):
+        got = [None, None]
+        errors = []
+
+        def work(i):
+            try:
+                (lo, hi) = parts[i]
+                stream = torch.cuda.Stream() if own_stream else torch.cuda.current_stream()
+                with torch.cuda.stream(stream):
+                    gq = Queue(hi - lo, ql, ql + ql * pv)
+                    gq.insert(gb[lo:hi], gd[lo:hi])
+                    t = closest_vectors(gv[lo:hi], gq, gv, gb, c, excluding_self(lo, hi))
+                    stream.synchronize()
+                got[i] = (t, host(gq.indices), host(gq.distances))
+            except Exception as e:  # surfaces in the main thread below
+                errors.append(e)
+
+        threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+        for th in threads:
+            th.start()
+        for th in threads:
+            th.join(timeout=120)
+        assert not any(th.is_alive() for th in threads), "a beam search did not return"
+        assert not errors, errors
+        for i in range(2):
+            (t_want, oq) = want[i]
+            assert got[i][0] == t_want
+            assert np.array_equal(got[i][1][:, :ql], oq.indices[:, :ql])
+            assert np.array_equal(bits(got[i][2][:, :ql]), bits(oq.distances[:, :ql]))
+
+
+def test_hand_enumerated_chain_on_the_gpu():
+    """The twelve-node chain of tests/test_oracle_search.py, whose trace is written out by hand there:
+    six iterations, nodes 11 and 10 at 1/16 and 2/16; eight nodes with node 6 excluded: four, nodes 7 and 5."""
+    say("hand-enumerated chain")
+    from vectorlink_gpu import Queue
+    from vectorlink_gpu.ann import BEAM_PER_QUERY_STOP, BEAM_SORT_MERGE, closest_vectors
+
+    c = cfg(beam_size=2, parallel_visit_count=1, visit_queue_factor=1, exclude_factor=2, speculative_readahead=1)
+    for (n, excl, flags, t_want, ids_want, d_want) in [
+            (12, None, 0, 6, [11, 10], [1 / 16, 2 / 16]), (12, None, BEAM_SORT_MERGE, 6, [11, 10], [1 / 16, 2 / 16]),
+            (8, None, 0, 4, [7, 6], [1 / 16, 2 / 16]), (8, [[6]], 0, 4, [7, 5], [1 / 16, 3 / 16]),
+            (12, None, BEAM_PER_QUERY_STOP, 5, [11, 10], [1 / 16, 2 / 16]),
+            (8, None, BEAM_PER_QUERY_STOP, 5, [7, 6], [1 / 16, 2 / 16])]:
+        delta = np.array([(n - i) / 16.0 for i in range(n)], dtype=np.float32)
+        v = (1.0 - 2.0 * delta).reshape(n, 1).astype(np.float32)
+        table = np.array([[(i + 1) % n, (i + 2) % n] for i in range(n)], dtype=np.int32)
+        q = Queue(1, 2, 4)
+        q.insert(dev(np.array([[0, 1]], dtype=np.int32)), dev(np.array([[delta[0], delta[1]]], dtype=np.float32)))
+        ex = None if excl is None else dev(np.array(excl, dtype=np.int32))
+        t = closest_vectors(dev(np.ones((1, 1), dtype=np.float32)), q, dev(v), dev(table), c, ex, flags=flags)
+        assert t == t_want, (n, excl, flags)
+        assert host(q.indices)[0, :2].tolist() == ids_want and host(q.distances)[0, :2].tolist() == d_want
+
+
+@pytest.mark.parametrize("n,dim,beam,bqf,pv,vqf,ef,ra", BEAM_CASES)
+def test_per_query_stop_against_its_model(n, dim, beam, bqf, pv, vqf, ef, ra):
+    """VL_BEAM_PER_QUERY_STOP against the CPU model that defines it (oracle.closest_vectors_per_query):
+    same iteration count, ids and distance bits, on a build step with self exclusion."""
+    say(f"per-query stop n={n} dim={dim} beam={beam}")
+    from vectorlink_gpu import Queue
+    from vectorlink_gpu.ann import BEAM_PER_QUERY_STOP, closest_vectors, excluding_self
+
+    rng = np.random.default_rng(1000 + n + dim)
+    v = unit(rng, n, dim)
+    c = cfg(beam_size=beam, beam_queue_factor=bqf, parallel_visit_count=pv, visit_queue_factor=vqf,
+            exclude_factor=ef, speculative_readahead=ra)
+    ql = beam * bqf
+    beams = orc.generate_circulant_beams(n, orc.primes(ql))
+    d = orc.calculate_distances(v, beams)
+    lo, hi = 3, n - 2
+    oq = orc.Queue(hi - lo, ql, ql + ql * pv)
+    oq.insert(beams[lo:hi], d[lo:hi])
+    t_want = orc.closest_vectors_per_query(v[lo:hi], oq, v, beams, c, orc.excluding_self(lo, hi))
+    gv, gb = dev(v), dev(beams)
+    gq = Queue(hi - lo, ql, ql + ql * pv)
+    gq.insert(gb[lo:hi], dev(d)[lo:hi])
+    t_got = closest_vectors(gv[lo:hi], gq, gv, gb, c, excluding_self(lo, hi), flags=BEAM_PER_QUERY_STOP)
+    assert t_got == t_want
+    assert np.array_equal(host(gq.indices)[:, :ql], oq.indices[:, :ql])
+    assert np.array_equal(bits(host(gq.distances)[:, :ql]), bits(oq.distances[:, :ql]))
+
+
+def test_per_query_stop_search_quality_and_cost():
+    """ANN.search(stop="per_query") equals its model on a built graph, needs no more iterations than the
+    reference's batch-wide stop needs, and loses little recall against it."""
+    say("per-query stop: search on a built graph")
+    from vectorlink_gpu import ANN
+
+    rng = np.random.default_rng(31)
+    n, dim = 6000, 48
+    v = unit(rng, n, dim)
+    qv = unit(rng, 500, dim)
+    kw = dict(beam_size=16, beam_queue_factor=2, recall_search_queue_factor=2, batch_size=2000, optimization_loops=2)
+    ann = ANN(dev(v), **kw)
+    c = cfg(**kw)
+    wb = host(ann.beams)
+    want = orc.search(v, wb, qv, c, stop="per_query")
+    got = ann.search(dev(qv), stop="per_query")
+    L = want.length
+    assert np.array_equal(host(got.indices)[:, :L], want.indices[:, :L])
+    assert np.array_equal(bits(host(got.distances)[:, :L]), bits(want.distances[:, :L]))
+    full = ann.search(dev(qv))
+    truth, _ = orc.knn_exact(qv, v, 10)
+
+    def recall(ids):
+        return np.mean([len(set(a[:10].tolist()) & set(t.tolist())) / 10 for a, t in zip(ids, truth)])
+
+    assert recall(host(got.indices)) > recall(host(full.indices)) - 0.05

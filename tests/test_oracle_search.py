@@ -163,3 +163,90 @@ def test_generate_ann_stale_distance_mode_differs_only_after_loop_zero():
     assert not np.array_equal(d1, d2)      # but the reference hands back the circulant distances
     init = orc.calculate_distances(v, orc.generate_circulant_beams(400, orc.primes(12)))
     assert np.array_equal(d2, init[:, :6])
+
+
+# ---- a beam search small enough to follow by hand ---------------------------------------------
+# One query q = [1.0] over one-dimensional "vectors" x_i = 1 - 2*delta_i, so that the distance of
+# node i is (1 - x_i) / 2 = delta_i exactly (sixteenths: no rounding anywhere).  Node i lists
+# [i+1, i+2] mod n and lies at delta_i = (n - i) / 16: every hop moves closer.  Configuration:
+# width 2, one visit per iteration, visit queue of 2 slots (+2 spare), visited list of 4 columns,
+# progress checked every iteration; search queue of 2 slots (+2 spare) seeded with nodes 0 and 1.
+#
+# n = 12, derived statement by statement from ann.py:66-91, queue.py:37-61,87-95, utils.py:61-82:
+#  it 1  pop 1    candidates 2,3    search [3,2|1,0]    visited [1]        visit [3,2|0,-]
+#  it 2  pop 3    candidates 4,5    search [5,4|3,2]    visited [1,3]      visit [5,4|2,-]   (0 is overwritten)
+#  it 3  pop 5    candidates 6,7    search [7,6|5,4]    visited [1,3,5]    visit [7,6|4,-]
+#  it 4  pop 7    candidates 8,9    search [9,8|7,6]    visited [1,3,5,7]  visit [9,8|6,-]
+#  it 5  pop 9    candidates 10,11  search [11,10|9,8]  no free column: add_new_to_seen_ returns None,
+#                                                       the visit queue is not fed and stays [-,8|6,-]
+#  it 6  pop -    (slot 0 was emptied by the pop of it 5 and nothing re-sorted the row: node 8 is never
+#                 visited)  no candidates, search prefix unchanged -> the loop ends.  T = 6.
+# n = 8: the visited list fills at it 4 ([1,3,5,7]); it 4 pops 7, candidates 0,1 leave the prefix
+#  [7,6] unchanged -> T = 4.  With node 6 excluded from the search queue (it still enters the visit
+#  queue, which only excludes visited nodes): it 3 gives search [7,5|4,-], it 4 changes nothing -> [7,5].
+def chain(n):
+    delta = np.array([(n - i) / 16.0 for i in range(n)], dtype=np.float32)
+    v = (1.0 - 2.0 * delta).reshape(n, 1).astype(np.float32)
+    beams = np.array([[(i + 1) % n, (i + 2) % n] for i in range(n)], dtype=np.int32)
+    c = cfg(beam_size=2, parallel_visit_count=1, visit_queue_factor=1, exclude_factor=2, speculative_readahead=1)
+    q = orc.Queue(1, 2, 4)
+    q.insert(np.array([[0, 1]], dtype=np.int32), np.array([[delta[0], delta[1]]], dtype=np.float32))
+    return v, beams, c, q, delta
+
+
+@pytest.mark.parametrize("loop", [orc.closest_vectors, orc.closest_vectors_py])
+def test_hand_enumerated_trace(loop):
+    one = np.ones((1, 1), dtype=np.float32)
+    v, beams, c, q, delta = chain(12)
+    assert loop(one, q, v, beams, c, None) == 6
+    assert q.indices[0, :2].tolist() == [11, 10]
+    assert q.distances[0, :2].tolist() == [1 / 16, 2 / 16]
+    v, beams, c, q, delta = chain(8)
+    assert loop(one, q, v, beams, c, None) == 4
+    assert q.indices[0, :2].tolist() == [7, 6] and q.distances[0, :2].tolist() == [1 / 16, 2 / 16]
+    v, beams, c, q, delta = chain(8)
+    assert loop(one, q, v, beams, c, np.array([[6]], dtype=np.int32)) == 4
+    assert q.indices[0, :2].tolist() == [7, 5] and q.distances[0, :2].tolist() == [1 / 16, 3 / 16]
+
+
+def test_hand_enumerated_trace_per_query_stop():
+    # the per-query model on the same chains.  n = 12: after every insert of it 1-4 the visit queue's
+    # head (3, 5, 7, 9) is closer than the search queue's last slot (2, 4, 6, 8), so the row goes on;
+    # at it 5 the visited list has no free column: the row stops, T = 5, same answer.  n = 8: at it 4
+    # head and last slot are both node 6 - not farther, so the row goes on; it 5 pops 6, its
+    # candidates 7 (queued already, collapsed as a neighbouring duplicate) and 0 change nothing, and
+    # the visited list is full: T = 5.
+    one = np.ones((1, 1), dtype=np.float32)
+    v, beams, c, q, delta = chain(12)
+    assert orc.closest_vectors_per_query(one, q, v, beams, c, None) == 5
+    assert q.indices[0, :2].tolist() == [11, 10]
+    v, beams, c, q, delta = chain(8)
+    assert orc.closest_vectors_per_query(one, q, v, beams, c, None) == 5
+    assert q.indices[0, :2].tolist() == [7, 6]
+
+
+def test_per_query_stop_rows_are_independent_and_no_worse_than_their_seeds():
+    # with a visited list that never fills, a row's result under the per-query stop depends on that row
+    # alone: the batch equals its rows searched one at a time; on a complete graph it is exact kNN
+    rng = np.random.default_rng(21)
+    n, dim = 400, 12
+    v = unit(rng, n, dim)
+    c = cfg(beam_size=6, beam_queue_factor=2, exclude_factor=40, speculative_readahead=3)
+    ql = 12
+    beams = orc.generate_circulant_beams(n, orc.primes(ql))
+    d = orc.calculate_distances(v, beams)
+    rows = slice(30, 70)
+    q = build_queue(v, beams, d, rows.start, rows.stop, ql, 4)
+    before = q.distances[:, :ql].copy()
+    t = orc.closest_vectors_per_query(v[rows], q, v, beams, c, orc.excluding_self(rows.start, rows.stop))
+    assert t % 3 == 0 and (q.distances[:, :ql] <= before).all()
+    for r in range(rows.start, rows.stop, 7):
+        one = build_queue(v, beams, d, r, r + 1, ql, 4)
+        orc.closest_vectors_per_query(v[r:r + 1], one, v, beams, c, orc.excluding_self(r, r + 1))
+        assert np.array_equal(one.indices[0, :ql], q.indices[r - rows.start, :ql])
+    full = np.stack([np.array([j for j in range(24) if j != i]) for i in range(24)]).astype(np.int32)
+    cc = cfg(beam_size=23, recall_search_queue_factor=1, parallel_visit_count=1, visit_queue_factor=1)
+    qv = unit(rng, 5, dim)
+    res = orc.search(v[:24], full, qv, cc, queue_size=4, stop="per_query")
+    want, _ = orc.knn_exact(qv, v[:24], 4)
+    assert np.array_equal(res.indices[:, :4], want)

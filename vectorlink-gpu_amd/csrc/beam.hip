@@ -21,6 +21,7 @@
 #include "rowsort.h"
 #include "dist_device.h"
 #include <stdlib.h>
+#include <mutex>
 
 int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors, int64_t n_vectors,
                      int64_t dim, const int32_t *ids, const int32_t *visit, int64_t n_visit,
@@ -40,7 +41,24 @@ struct BeamProfile {
     double expand_ms = 0, merge_ms = 0;
     int64_t expand_launches = 0, merge_launches = 0, evals = 0, rows = 0, iterations = 0, wanted = 0;
 };
+// The only mutable state of the library besides the thread-local error text.  A call
+// sums into a BeamProfile of its own and adds it here once, under the mutex, when it
+// returns, so calls on different host threads do not tear each other's sums.
 BeamProfile g_prof;
+std::mutex g_prof_mutex;
+
+// HIP events of one profiled call; destroyed on every way out of the call.
+struct EventSet {
+    hipEvent_t ev[3 * 64];
+    int n = 0;
+    int create(int count) {
+        for (; n < count; ++n) VL_HIP(hipEventCreate(&ev[n]));
+        return VL_OK;
+    }
+    ~EventSet() {
+        for (int i = 0; i < n; ++i) (void)hipEventDestroy(ev[i]);
+    }
+};
 
 struct MergeArgs {
     BeamCtrl *ctrl;
@@ -61,6 +79,7 @@ struct MergeArgs {
     int32_t *seen;
     int32_t *seen_count;
     int E;
+    int32_t *row_done;  // per-query stop only (else null): 1 once a row has stopped expanding
 };
 
 __device__ inline bool sorted_contains(const int32_t *a, int n, int32_t v) {
@@ -90,7 +109,8 @@ __global__ void beam_memo_clear_kernel(uint64_t *memo, int64_t n) {
 
 __global__ __launch_bounds__(kQueueThreads) void beam_init_kernel(BeamCtrl *ctrl, int64_t n_rows, const int32_t *q_ids,
                                                                  const float *q_d, int cap, int head, int32_t *v_ids,
-                                                                 float *v_d, int VL, int32_t *seen_count) {
+                                                                 float *v_d, int VL, int32_t *seen_count,
+                                                                 int32_t *row_done) {
     int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t == 0) {
         ctrl->stop = 0;
@@ -102,7 +122,10 @@ __global__ __launch_bounds__(kQueueThreads) void beam_init_kernel(BeamCtrl *ctrl
         ctrl->evals[t] = 0;
         ctrl->wanted[t] = 0;
     }
-    if (t < n_rows) seen_count[t] = 0;
+    if (t < n_rows) {
+        seen_count[t] = 0;
+        row_done[t] = 0;
+    }
     if (t < n_rows * VL) {  // Queue.initialize_from_queue, queue.py:30-35
         int64_t r = t / VL;
         int i = (int)(t % VL);
@@ -198,7 +221,7 @@ __global__ __launch_bounds__(kQueueThreads) void beam_merge_kernel(MergeArgs a) 
     for (int i = threadIdx.x; i < cnt; i += blockDim.x) seen_a[i] = srow[i];
     if (threadIdx.x == 0) n_new_s = 0;
     __syncthreads();
-    const int n_add = min(a.E - first, a.Vt);  // utils.py:73-75
+    const int n_add = min(min(a.E - first, a.Vt), a.E - cnt);  // utils.py:73-75 (cnt <= first: rows are packed)
     if (threadIdx.x < kWave) {
         const int j = threadIdx.x;
         int32_t x = j < n_add ? vrow_i[j] : VL_MAXINT;
@@ -352,6 +375,7 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
     __shared__ int n_ex_s;
     __shared__ int32_t newv[kMaxVisit];
     __shared__ int n_new_s;
+    __shared__ uint64_t tail_s;  // per-query stop: the key that ends up in the search queue's last slot
 
     // Every global read of this workgroup is issued up front, before any of them
     // is waited for: the control words, the candidates, both queues, the popped
@@ -417,7 +441,7 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
 
     // ---- add_new_to_seen_ : utils.py:61-82 (does not depend on the candidates) ------
     if (!seen_full) {
-        const int n_add = min(a.E - first, a.Vt);
+        const int n_add = min(min(a.E - first, a.Vt), a.E - cnt);  // cnt <= first: rows are packed
         if (threadIdx.x < kWave) {
             const int j = threadIdx.x;
             int32_t x = j < n_add ? popped : VL_MAXINT;
@@ -521,6 +545,7 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
                 qi[r] = vl_key_id(k);
                 qd[r] = vl_key_dist(k);
             }
+            if (r == a.L - 1) tail_s = k;
         }
         for (int j = threadIdx.x; j < n_s; j += blockDim.x) {
             uint64_t k = cc[j];
@@ -530,15 +555,21 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
                 qd[r] = vl_key_dist(k);
                 diff = true;  // a new id inside the first L slots: the row changed (queue.py:57-59)
             }
+            if (r == a.L - 1) tail_s = k;
         }
     }
-    if (checking && __ballot(diff) && lane == 0) {
-        int *flag = &c->changed[(t / a.readahead) & 63];  // every writer stores the same 1: no atomic needed
+    int *flag = &c->changed[(t / a.readahead) & 63];  // every writer stores the same 1: no atomic needed
+    if (!a.row_done && checking && __ballot(diff) && lane == 0) {
         if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
             __hip_atomic_store(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (seen_full) return;
+    if (seen_full) {
+        // no pop yields a real id from now on: with the per-query stop the row is finished
+        if (a.row_done && threadIdx.x == 0) a.row_done[row] = 1;
+        return;
+    }
     __syncthreads();  // cc is reused below
+    const uint64_t tail = n_s ? tail_s : ws;
 
     // ---- visit_queue.insert(candidates, exclude=seen) : ann.py:85-88 --------------------
     auto keep_visit = [&](int i) -> bool {
@@ -569,6 +600,17 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
     for (int r = nva + n_v + threadIdx.x; r < a.VL; r += blockDim.x) {  // the popped slots end up here, empty
         vi[r] = VL_MAXINT;
         vd[r] = VL_MAXFLOAT;
+    }
+    if (a.row_done && threadIdx.x == 0) {
+        // Per-query stop: the row is finished when the best node it has not visited yet is farther than the
+        // last slot of its search queue (or nothing is left to visit); otherwise it keeps the loop going.
+        uint64_t head = kPadKey;
+        if (nva > 0) head = va[0];
+        if (n_v > 0 && cc[0] < head) head = cc[0];
+        const bool done = head == kPadKey || vl_key_id(head) == VL_MAXINT || head > tail;
+        if (done) a.row_done[row] = 1;
+        else if (checking && __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
+            __hip_atomic_store(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
@@ -604,8 +646,9 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
     const int gate = beam_gate(c, t, a.readahead, a.E, blockIdx.x == 0 && threadIdx.x == 0);
     if (gate == 2) return;
     const int64_t row = blockIdx.x;
-    if (gate == 1) {
-        // the visit queue is no longer fed: every candidate of this iteration is empty
+    if (gate == 1 || (a.row_done && a.row_done[row])) {
+        // the visit queue is no longer fed (every candidate of this iteration is empty), or this row has
+        // stopped on its own: nothing changes, only the running maximum is kept current
         if (threadIdx.x == 0) raise_running_max(&c->first[(t + 1) % 3], a.seen_count[row], min(a.E, a.Vt * t));
         return;
     }
@@ -685,7 +728,7 @@ int launch_step_by_dim(const StepArgs &s, bool aligned, int threads, size_t smem
 
 struct BeamLayout {
     int64_t m, VL, Vt, E, head;
-    int64_t off_cand_ids, off_cand_d, off_v_ids, off_v_d, off_seen, off_seen_count, off_ctrl, off_memo, total;
+    int64_t off_cand_ids, off_cand_d, off_v_ids, off_v_d, off_seen, off_seen_count, off_row_done, off_ctrl, off_memo, total;
     int memo_slots;
 };
 
@@ -720,6 +763,7 @@ int beam_layout(const vl_beam_params *p, BeamLayout *l) {
     l->off_v_d = o; o = align256(o + p->n_rows * l->VL * 4);
     l->off_seen = o; o = align256(o + p->n_rows * l->E * 4);
     l->off_seen_count = o; o = align256(o + p->n_rows * 4);
+    l->off_row_done = o; o = align256(o + p->n_rows * 4);
     l->off_ctrl = o; o = align256(o + (int64_t)sizeof(BeamCtrl));
     // per-row cache of evaluated (id, distance) pairs: 128 slots per candidate of one iteration,
     // 1Ki..64Ki per row, the whole table at most 8 GiB (measured at 1M x 768: 16Ki -> 64Ki slots cuts the
@@ -773,6 +817,7 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
     float *v_d = (float *)(ws + l.off_v_d);
     int32_t *seen = (int32_t *)(ws + l.off_seen);
     int32_t *seen_count = (int32_t *)(ws + l.off_seen_count);
+    int32_t *row_done = (int32_t *)(ws + l.off_row_done);
     BeamCtrl *ctrl = (BeamCtrl *)(ws + l.off_ctrl);
 
     {
@@ -781,7 +826,7 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
         if (n < p->n_rows) n = p->n_rows;
         hipLaunchKernelGGL(beam_init_kernel, dim3((unsigned)((n + kQueueThreads - 1) / kQueueThreads)),
                            dim3(kQueueThreads), 0, st, ctrl, p->n_rows, q_ids, q_dists, (int)p->queue_capacity,
-                           (int)l.head, v_ids, v_d, (int)l.VL, seen_count);
+                           (int)l.head, v_ids, v_d, (int)l.VL, seen_count, row_done);
         VL_LAUNCH_CHECK("beam_init_kernel");
     }
     uint64_t *memo = (uint64_t *)(ws + l.off_memo);
@@ -798,6 +843,8 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
     a.excl = p->excl_cols > 0 ? exclude : nullptr; a.excl_cols = a.excl ? (int)p->excl_cols : 0;
     a.v_ids = v_ids; a.v_d = v_d; a.VL = (int)l.VL; a.Vt = (int)l.Vt; a.Pv = vl_next_pow2(l.VL + l.m);
     a.seen = seen; a.seen_count = seen_count; a.E = (int)l.E;
+    const bool per_query = (p->flags & VL_BEAM_PER_QUERY_STOP) != 0;
+    a.row_done = per_query ? row_done : nullptr;
     a.Pc = vl_next_pow2(l.m);
     if (a.Pc < 2) a.Pc = 2;
     // VL_BEAM_MERGE=sort selects the full-row-sort form of the merge step (exact for queue rows in any state)
@@ -825,6 +872,7 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
         return !(e && e[0] == '0');
     }();
     const bool use_fused = fused_env && !use_sort_merge && merge_threads != 64 && !(p->flags & VL_BEAM_TWO_LAUNCHES);
+    VL_REQUIRE(!per_query || use_fused, "the per-query stop is only built into the fused step");
     const bool aligned = (p->dim % 4 == 0) && (((uintptr_t)queries | (uintptr_t)vectors) % 16 == 0);
     StepArgs step;
     step.queries = queries; step.vectors = vectors; step.beams = beams; step.n_vectors = p->n_vectors;
@@ -838,13 +886,25 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
         step.memo_shift = 32 - lg;
     }
     const int R = (int)p->speculative_readahead;
-    const bool prof = g_prof.enabled != 0;
+    bool prof;
+    {
+        std::lock_guard<std::mutex> hold(g_prof_mutex);
+        prof = g_prof.enabled != 0;
+    }
     step.count_evals = prof ? 1 : 0;
-    hipEvent_t ev[3 * 64];
+    EventSet events;
+    hipEvent_t *ev = events.ev;
+    BeamProfile mine;
     if (prof) {
         VL_REQUIRE(R <= 64, "profiling supports speculative_readahead up to 64");
-        for (int i = 0; i < 3 * R; ++i) VL_HIP(hipEventCreate(&ev[i]));
+        rc = events.create(3 * R);
+        if (rc < 0) return rc;
     }
+    // A row expands real nodes in an unbroken run of iterations from the first one, each of
+    // which adds at least one id to its visited list of E slots; once no row expands, no
+    // queue changes and the next check ends the loop.  More iterations than that mean the
+    // control block was overwritten while the loop ran (a workspace shared by two calls).
+    const int64_t t_limit = l.E + l.VL + 2 * (int64_t)R + 2;
     int64_t t = 0;
     for (;;) {
         for (int r = 0; r < R; ++r) {
@@ -881,29 +941,37 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
             for (int r = 0; r < R; ++r) {
                 float ms = 0;
                 VL_HIP(hipEventElapsedTime(&ms, ev[3 * r], ev[3 * r + 1]));
-                g_prof.expand_ms += ms;
+                mine.expand_ms += ms;
                 if (!use_fused) {
                     VL_HIP(hipEventElapsedTime(&ms, ev[3 * r + 1], ev[3 * r + 2]));
-                    g_prof.merge_ms += ms;
+                    mine.merge_ms += ms;
                 }
             }
-            g_prof.expand_launches += R;
-            g_prof.merge_launches += R;
+            mine.expand_launches += R;
+            mine.merge_launches += R;
         }
         if (!changed) break;  // ann.py:90-91
-        VL_REQUIRE(t < (1ll << 30), "beam search did not terminate");
+        if (t > t_limit) {
+            vl_set_error("beam search still changing after %lld iterations (bound %lld): its workspace was "
+                         "overwritten while it ran - is it shared with a concurrent call?",
+                         (long long)t, (long long)t_limit);
+            return VL_ERR_STATE;
+        }
     }
     if (prof) {
-        static thread_local unsigned long long ev_counts[kBeamStripes];
+        unsigned long long ev_counts[kBeamStripes];
         VL_HIP(hipMemcpyAsync(ev_counts, ctrl->evals, sizeof(ev_counts), hipMemcpyDeviceToHost, st));
         VL_HIP(hipStreamSynchronize(st));
-        for (int i = 0; i < kBeamStripes; ++i) g_prof.evals += (int64_t)ev_counts[i];
+        for (int i = 0; i < kBeamStripes; ++i) mine.evals += (int64_t)ev_counts[i];
         VL_HIP(hipMemcpyAsync(ev_counts, ctrl->wanted, sizeof(ev_counts), hipMemcpyDeviceToHost, st));
         VL_HIP(hipStreamSynchronize(st));
-        for (int i = 0; i < kBeamStripes; ++i) g_prof.wanted += (int64_t)ev_counts[i];
+        for (int i = 0; i < kBeamStripes; ++i) mine.wanted += (int64_t)ev_counts[i];
+        std::lock_guard<std::mutex> hold(g_prof_mutex);
+        g_prof.expand_ms += mine.expand_ms; g_prof.merge_ms += mine.merge_ms;
+        g_prof.expand_launches += mine.expand_launches; g_prof.merge_launches += mine.merge_launches;
+        g_prof.evals += mine.evals; g_prof.wanted += mine.wanted;
         g_prof.rows += p->n_rows;
         g_prof.iterations += t;
-        for (int i = 0; i < 3 * R; ++i) (void)hipEventDestroy(ev[i]);
     }
     return t;
 }
@@ -915,6 +983,7 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
 // candidate distances asked for (fetched + served by the per-row cache),
 // summed since the last reset.
 VL_EXPORT int vl_beam_profile(int enable, int reset, double *out) {
+    std::lock_guard<std::mutex> hold(g_prof_mutex);
     if (out) {
         out[0] = g_prof.expand_ms; out[1] = g_prof.merge_ms;
         out[2] = (double)g_prof.expand_launches; out[3] = (double)g_prof.merge_launches;

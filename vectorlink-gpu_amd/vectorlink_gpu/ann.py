@@ -6,6 +6,7 @@ to libvlgpu.so.  Differences are stated where they occur.
 from __future__ import annotations
 
 import ctypes
+import threading
 import time
 from typing import Dict, Optional, Tuple
 
@@ -22,6 +23,7 @@ from .utils import add_new_to_seen_, generate_circulant_beams, generate_queue_ci
 
 BEAM_TWO_LAUNCHES = 1  # include/vlgpu.h: VL_BEAM_TWO_LAUNCHES
 BEAM_SORT_MERGE = 2    # include/vlgpu.h: VL_BEAM_SORT_MERGE
+BEAM_PER_QUERY_STOP = 4  # include/vlgpu.h: VL_BEAM_PER_QUERY_STOP (a different loop: every row stops on its own)
 
 
 def _beam_params(batch: int, dim: int, n_vectors: int, width: int, queue: Queue, config: Dict,
@@ -34,15 +36,36 @@ def _beam_params(batch: int, dim: int, n_vectors: int, width: int, queue: Queue,
         excl_cols=excl_cols, flags=flags)
 
 
-_WORKSPACES: Dict[str, Tensor] = {}
+class _Workspace:
+    """Scratch memory of the beam-search loop for one (device, stream): the loop's control
+    block, visit queues, visited lists and distance cache live in it, so two calls must
+    never share it while either runs.  The lock serialises host threads that launch on the
+    same stream; calls on different streams get different workspaces and may overlap."""
+
+    def __init__(self):
+        self.lock = threading.Lock()
+        self.tensor: Optional[Tensor] = None
+
+    def reserve(self, nbytes: int, device) -> Tensor:
+        if self.tensor is None or self.tensor.numel() < nbytes:
+            self.tensor = None  # let the old block go before the larger one is asked for
+            self.tensor = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        return self.tensor
 
 
-def _workspace(nbytes: int, device) -> Tensor:
-    """One growing scratch tensor per device, owned by torch's allocator."""
-    key = str(device)
-    ws = _WORKSPACES.get(key)
-    if ws is None or ws.numel() < nbytes:
-        _WORKSPACES[key] = ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+_WORKSPACES: Dict[Tuple[str, int], _Workspace] = {}
+_WORKSPACES_LOCK = threading.Lock()
+
+
+def _workspace(device) -> _Workspace:
+    """The workspace of torch's current stream on `device` (owned by torch's allocator)."""
+    dev = torch.device(device)
+    index = dev.index if dev.index is not None else torch.cuda.current_device()
+    key = (f"cuda:{index}", int(torch.cuda.current_stream(index).cuda_stream))
+    with _WORKSPACES_LOCK:
+        ws = _WORKSPACES.get(key)
+        if ws is None:
+            _WORKSPACES[key] = ws = _Workspace()
     return ws
 
 
@@ -87,7 +110,15 @@ def closest_vectors(query_vecs: Tensor, search_queue: Queue, vectors: Tensor, be
     """reference ann.py:38-93.  Updates search_queue in place; returns the
     number of iterations run (the reference returns True).  Rows are exact on
     [:, :search_queue.length]; the slots beyond are unspecified.  flags picks
-    another form of the same loop (BEAM_TWO_LAUNCHES, BEAM_SORT_MERGE)."""
+    another form of the same loop (BEAM_TWO_LAUNCHES, BEAM_SORT_MERGE) or the
+    per-query stop (BEAM_PER_QUERY_STOP: not the reference's loop, which keeps
+    every row expanding until the whole batch is quiet, ann.py:90-91).
+
+    The default form relies on what Queue.insert leaves behind: rows ordered by
+    (distance, id) with distinct ids, and an id carrying the same distance
+    wherever it occurs, i.e. the queue's distances are distances to `vectors`
+    rows under this call's query rows.  For a queue in any other state pass
+    BEAM_SORT_MERGE, which sorts whole rows like the reference does."""
     assert query_vecs.dtype == torch.float32 and vectors.dtype == torch.float32 and beams.dtype == torch.int32
     nv.require_gpu(query_vecs, vectors, beams, search_queue.indices, exclude)
     query_vecs = query_vecs.contiguous()
@@ -102,10 +133,12 @@ def closest_vectors(query_vecs: Tensor, search_queue: Queue, vectors: Tensor, be
     p = _beam_params(batch, dim, vectors.size(0), beams.size(1), search_queue, config,
                      0 if excl is None else excl.size(1), flags)
     need = nv.check(nv.lib().vl_beam_workspace_bytes(ctypes.byref(p)))
-    ws = _workspace(need, vectors.device)
-    iterations = nv.check(nv.lib().vl_closest_vectors(
-        ctypes.byref(p), nv.ptr(query_vecs), nv.ptr(vectors), nv.ptr(beams), nv.ptr(search_queue.indices),
-        nv.ptr(search_queue.distances), nv.ptr(excl), nv.ptr(ws), ws.numel(), nv.stream()))
+    workspace = _workspace(vectors.device)
+    with workspace.lock:
+        ws = workspace.reserve(need, vectors.device)
+        iterations = nv.check(nv.lib().vl_closest_vectors(
+            ctypes.byref(p), nv.ptr(query_vecs), nv.ptr(vectors), nv.ptr(beams), nv.ptr(search_queue.indices),
+            nv.ptr(search_queue.distances), nv.ptr(excl), nv.ptr(ws), ws.numel(), nv.stream()))
     return iterations
 
 
@@ -127,7 +160,11 @@ class GraphBuild:
     reference's behaviour (and then uses the step-by-step loop, because the
     fused loop relies on an id always carrying the same distance)."""
 
-    def __init__(self, vectors: Tensor, config: Dict, stale_distances: bool = False):
+    def __init__(self, vectors: Tensor, config: Dict, stale_distances: bool = False,
+                 initial: Optional[Tuple[Tensor, Tensor]] = None, keep_history: bool = False):
+        """initial: (ids, distances) tables of the build-queue width to start from instead of the
+        circulant graph (a later optimisation loop's starting state).  keep_history: keep a
+        reference to the tables every optimisation loop started from in self.history."""
         self.vectors = vectors
         self.config = config
         self.stale = stale_distances
@@ -135,11 +172,16 @@ class GraphBuild:
         device = vectors.device
         self.beam_size = config["beam_size"]
         self.queue_length = self.beam_size * config["beam_queue_factor"]
-        neighbor_primes = primes(self.queue_length, device)
-        self.beams = generate_circulant_beams(self.num_vecs, neighbor_primes)
-        self.beam_distances = calculate_distances(vectors, self.beams)  # of the circulant graph
+        if initial is None:
+            neighbor_primes = primes(self.queue_length, device)
+            self.beams = generate_circulant_beams(self.num_vecs, neighbor_primes)
+            self.beam_distances = calculate_distances(vectors, self.beams)  # of the circulant graph
+        else:
+            (self.beams, self.beam_distances) = initial
+            assert self.beams.size() == (self.num_vecs, self.queue_length) == self.beam_distances.size()
         self.distances = self.beam_distances
         self.stats: list = []  # one dict per finished optimisation loop
+        self.history: Optional[list] = [] if keep_history else None
         self.finished = False
 
     def batches_per_loop(self) -> int:
@@ -156,6 +198,8 @@ class GraphBuild:
         for loop in range(0, config["optimization_loops"]):
             loop_start = time.time()
             iterations = 0
+            if self.history is not None:
+                self.history.append((self.beams, self.beam_distances if self.stale else self.distances))
             next_beams = torch.empty_like(self.beams)
             next_beam_distances = torch.empty_like(self.beam_distances)
             for start in range(0, self.num_vecs, batch_size):
@@ -477,11 +521,17 @@ class ANN:
             self._entry = (ids, self.vectors[ids.long()].contiguous())
         return self._entry
 
-    def search(self, query: Tensor, queue_size: Optional[int] = None, seeding: Optional[str] = None) -> Queue:
+    def search(self, query: Tensor, queue_size: Optional[int] = None, seeding: Optional[str] = None,
+               stop: str = "batch") -> Queue:
         """reference ann.py:469-477: takes a batch of query vectors, returns the
         search Queue; the answer is queue.indices[:, :k] / queue.distances[:, :k].
         queue_size overrides the configured search-queue length, seeding the
-        instance's seeding mode."""
+        instance's seeding mode.  stop="batch" is the reference's loop (every row
+        expands until no row of the batch changed at a progress check);
+        stop="per_query" ends each row on its own once its best unvisited node is
+        farther than the last slot of its queue - faster for large batches, not
+        the reference's result."""
+        assert stop in ("batch", "per_query")
         assert query.dim() == 2 and query.dtype == torch.float32
         if not query.is_cuda:
             query = query.to(self.vectors.device)
@@ -494,7 +544,8 @@ class ANN:
                                               queue_size)
         else:
             search_queue = initial_search_queue(self.vectors, query, self.configuration, queue_size)
-        closest_vectors(query, search_queue, self.vectors, self.beams, self.configuration, None)
+        closest_vectors(query, search_queue, self.vectors, self.beams, self.configuration, None,
+                        flags=BEAM_PER_QUERY_STOP if stop == "per_query" else 0)
         return search_queue
 
     def recall_at_k(self, query: Tensor, k: int = 10, queue_size: Optional[int] = None,
