@@ -54,6 +54,14 @@ int vl_version(void);
 
 /* ---- distances -------------------------------------------------------- */
 
+/* The reference has one metric, the cosine distance of unit rows
+ * clamp((1 - <a, b>) / 2, 0, 1) (kernels.py:85-114).  VL_METRIC_L2 is an
+ * addition: the squared Euclidean distance sum_j (a_j - b_j)^2, not clamped,
+ * accumulated in the same order (for unit rows it equals 4 x the cosine
+ * distance up to rounding, so both order neighbours alike). */
+#define VL_METRIC_COSINE 0
+#define VL_METRIC_L2 1
+
 /* out[r, j] = clamp((1 - <queries[r], vectors[ids[r, j]]>) / 2, 0, 1);
  * VL_MAXFLOAT where ids[r, j] is VL_MAXINT or outside [0, n_vectors).
  * With queries == vectors and ids == beams this is calculate_distances
@@ -64,6 +72,12 @@ int vl_gather_distances(const float *queries, int64_t n_rows,
                         const int32_t *ids, int64_t width,
                         float *out, void *stream);
 
+/* vl_gather_distances with the metric chosen by the caller (VL_METRIC_*). */
+int vl_gather_distances_metric(const float *queries, int64_t n_rows,
+                               const float *vectors, int64_t n_vectors, int64_t dim,
+                               const int32_t *ids, int64_t width, int metric,
+                               float *out, void *stream);
+
 /* search_from_seeds (kernels.py:260-311, kernel 204-257): for row b, visit
  * slot s, neighbour slot k: nb = beams[visit[b,s], k];
  * idx_out[b, s*width+k] = nb, dist_out[...] = d(vectors[nb], queries[b]).
@@ -73,6 +87,13 @@ int vl_search_from_seeds(const float *queries, int64_t n_rows, int64_t dim,
                          const int32_t *beams, int64_t n_nodes, int64_t width,
                          const float *vectors, int64_t n_vectors,
                          int32_t *idx_out, float *dist_out, void *stream);
+
+/* vl_search_from_seeds with the metric chosen by the caller (VL_METRIC_*). */
+int vl_search_from_seeds_metric(const float *queries, int64_t n_rows, int64_t dim,
+                                const int32_t *visit, int64_t n_visit,
+                                const int32_t *beams, int64_t n_nodes, int64_t width,
+                                const float *vectors, int64_t n_vectors, int metric,
+                                int32_t *idx_out, float *dist_out, void *stream);
 
 /* ---- seed graphs ------------------------------------------------------ */
 
@@ -155,6 +176,7 @@ typedef struct vl_beam_params {
     int64_t speculative_readahead;
     int64_t excl_cols;            /* columns of the exclusion tensor, 0 if none */
     int64_t flags;                /* 0 = default; VL_BEAM_* bits select another form of the same loop */
+    int64_t metric;               /* VL_METRIC_COSINE (the reference's) or VL_METRIC_L2 */
 } vl_beam_params;
 
 /* Forms of one iteration, all with the same result on [:, :queue_length]:
@@ -167,12 +189,13 @@ typedef struct vl_beam_params {
 /* A different loop, not the reference's: PER_QUERY_STOP ends every row on its
  * own.  The reference tests for progress over the whole batch (ann.py:90-91),
  * so every row keeps expanding until the slowest one is quiet.  With this bit a
- * row stops expanding once the best node it has not visited yet is farther
- * than the last slot of its search queue (or nothing is left to visit), later
- * iterations skip it, and the loop ends at the first progress check that finds
- * every row stopped.  Results differ from the reference's loop (fewer
- * expansions per row); they are defined by, and tested against, the CPU model
- * closest_vectors_per_query of the test oracle.  Fused step only. */
+ * row is finished after speculative_readahead iterations in a row that left
+ * the first queue_length ids of its search queue unchanged (or when the visited
+ * list has no free column), later iterations skip it, and the loop ends at the
+ * first progress check that finds every row finished.  Results differ from the
+ * reference's loop (fewer expansions per row); they are defined by, and tested
+ * against, the CPU model closest_vectors_per_query of the test oracle.  Fused
+ * step only. */
 #define VL_BEAM_PER_QUERY_STOP 4
 
 int64_t vl_beam_workspace_bytes(const vl_beam_params *p);

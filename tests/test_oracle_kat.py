@@ -404,3 +404,66 @@ def test_rank_prune_and_reverse_merge_against_models():
                 real = merged[x][merged[x] != M]
                 assert len(set(real.tolist())) == len(real) and x not in real.tolist()
                 assert merged[x, :keep].tolist()[:int((got[x, :keep] != M).sum())] == got[x, :keep][got[x, :keep] != M].tolist()
+
+
+# ---------------------------------------------------------------- squared L2 (an addition: not in the reference)
+def test_l2_known_answers():
+    a = np.array([3, 0, -1, 2, 5], np.float32)
+    b = np.ones(5, np.float32)
+    assert orc.l2(a, b) == 26.0 and orc.l2(b, a) == 26.0          # 4 + 1 + 4 + 1 + 16
+    assert orc.l2(a, a) == 0.0
+    e0 = np.zeros(8, np.float32); e0[0] = 1
+    e1 = np.zeros(8, np.float32); e1[1] = 1
+    assert orc.l2(e0, e1) == 2.0 and orc.l2(e0, -e0) == 4.0        # orthogonal, antipodal unit vectors
+    big = np.full(4, 100.0, np.float32)
+    assert orc.l2(big, -big) == 160000.0                           # no clamp to [0, 1]
+
+
+@pytest.mark.parametrize("dim", [1, 3, 4, 5, 63, 64, 128, 255, 257, 384, 768, 1030, 1536, 2049])
+def test_l2_against_float64_and_cosine(dim):
+    rng = np.random.default_rng(900 + dim)
+    for _ in range(10):
+        a = rng.standard_normal(dim).astype(np.float32)
+        b = rng.standard_normal(dim).astype(np.float32) * 3
+        want = np.sum((a.astype(np.float64) - b.astype(np.float64)) ** 2)
+        assert abs(float(orc.l2(a, b)) - want) <= 1e-5 * want
+        assert orc.l2(a, b) == orc.l2(b, a)
+        # on unit rows |a - b|^2 = 2 - 2<a, b> = 4 x the cosine distance
+        a /= np.linalg.norm(a); b /= np.linalg.norm(b)
+        assert abs(float(orc.l2(a, b)) - 4 * float(orc.distance(a, b))) < 2e-6
+
+
+@pytest.mark.parametrize("dim", [5, 130, 771])
+def test_l2_every_element_counts(dim):
+    # a dropped, doubled or misplaced element, or a difference taken crosswise, changes an exact sum
+    for i in range(dim):
+        a = np.zeros(dim, np.float32); b = np.zeros(dim, np.float32)
+        a[i] = 3.0; b[i] = 0.5
+        assert orc.l2(a, b) == np.float32(6.25)
+    a = np.arange(1, dim + 1, dtype=np.float32)
+    assert orc.l2(a, np.zeros(dim, np.float32)) == np.float32(dim * (dim + 1) * (2 * dim + 1) / 6)
+    assert orc.l2(a, a - 2) == np.float32(4 * dim)
+
+
+def test_l2_metric_switch_reaches_the_drivers_and_is_restored():
+    rng = np.random.default_rng(5)
+    v = rng.standard_normal((60, 12)).astype(np.float32)
+    ids = rng.integers(0, 60, (60, 5)).astype(np.int32)
+    ids[4, 1] = M
+    cos = orc.calculate_distances(v, ids)
+    with orc.metric("l2"):
+        out = orc.calculate_distances(v, ids)
+        for r, c in itertools.product(range(60), range(5)):
+            if ids[r, c] == M:
+                assert out[r, c] == F
+            else:
+                assert out[r, c] == orc.l2(v[ids[r, c]], v[r])
+        # a complete graph searched by L2 returns the exact L2 neighbours (not the cosine ones: rows differ in length)
+        full = np.stack([np.array([j for j in range(24) if j != i]) for i in range(24)]).astype(np.int32)
+        c = dict(orc.DEFAULT_CONFIG, beam_size=23, recall_search_queue_factor=1, parallel_visit_count=1,
+                 visit_queue_factor=1)
+        q = rng.standard_normal((6, 12)).astype(np.float32)
+        res = orc.search(v[:24], full, q, c, queue_size=4)
+        d2 = ((q[:, None, :].astype(np.float64) - v[None, :24, :]) ** 2).sum(2)
+        assert np.array_equal(res.indices[:, :4], np.argsort(d2, axis=1, kind="stable")[:, :4])
+    assert np.array_equal(orc.calculate_distances(v, ids), cos)

@@ -210,18 +210,22 @@ def test_hand_enumerated_trace(loop):
 
 
 def test_hand_enumerated_trace_per_query_stop():
-    # the per-query model on the same chains.  n = 12: after every insert of it 1-4 the visit queue's
-    # head (3, 5, 7, 9) is closer than the search queue's last slot (2, 4, 6, 8), so the row goes on;
-    # at it 5 the visited list has no free column: the row stops, T = 5, same answer.  n = 8: at it 4
-    # head and last slot are both node 6 - not farther, so the row goes on; it 5 pops 6, its
-    # candidates 7 (queued already, collapsed as a neighbouring duplicate) and 0 change nothing, and
-    # the visited list is full: T = 5.
+    # the per-query model on the same chains, patience = speculative_readahead = 1.  n = 12: iterations
+    # 1-5 each change the search queue; at it 5 the visited list has no free column, the row is
+    # finished: T = 5, same answer.  n = 8: it 4 leaves the prefix [7,6] unchanged -> finished, T = 4.
+    # With patience 2 (progress checked every second iteration) on n = 8: it 4 is the first quiet
+    # iteration, it 5 pops 6 (candidates 7 and 0 change nothing) and the visited list is full: T = 6,
+    # the first check at which the row is finished.
     one = np.ones((1, 1), dtype=np.float32)
     v, beams, c, q, delta = chain(12)
     assert orc.closest_vectors_per_query(one, q, v, beams, c, None) == 5
     assert q.indices[0, :2].tolist() == [11, 10]
     v, beams, c, q, delta = chain(8)
-    assert orc.closest_vectors_per_query(one, q, v, beams, c, None) == 5
+    assert orc.closest_vectors_per_query(one, q, v, beams, c, None) == 4
+    assert q.indices[0, :2].tolist() == [7, 6]
+    v, beams, c, q, delta = chain(8)
+    c["speculative_readahead"] = 2
+    assert orc.closest_vectors_per_query(one, q, v, beams, c, None) == 6
     assert q.indices[0, :2].tolist() == [7, 6]
 
 

@@ -28,7 +28,7 @@ int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors,
                      const int32_t *beams, int64_t n_nodes, int64_t width, int64_t m,
                      int32_t *idx_out, float *dist_out, BeamCtrl *ctrl, int iter, int readahead,
                      int seen_cols, int64_t visit_stride, int count_evals, uint64_t *memo, int memo_slots,
-                     hipStream_t st);
+                     int metric, hipStream_t st);
 
 namespace {
 
@@ -79,7 +79,7 @@ struct MergeArgs {
     int32_t *seen;
     int32_t *seen_count;
     int E;
-    int32_t *row_done;  // per-query stop only (else null): 1 once a row has stopped expanding
+    int32_t *row_quiet;  // per-query stop only (else null): iterations in a row that left the row's search queue unchanged
 };
 
 __device__ inline bool sorted_contains(const int32_t *a, int n, int32_t v) {
@@ -110,7 +110,7 @@ __global__ void beam_memo_clear_kernel(uint64_t *memo, int64_t n) {
 __global__ __launch_bounds__(kQueueThreads) void beam_init_kernel(BeamCtrl *ctrl, int64_t n_rows, const int32_t *q_ids,
                                                                  const float *q_d, int cap, int head, int32_t *v_ids,
                                                                  float *v_d, int VL, int32_t *seen_count,
-                                                                 int32_t *row_done) {
+                                                                 int32_t *row_quiet) {
     int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t == 0) {
         ctrl->stop = 0;
@@ -124,7 +124,7 @@ __global__ __launch_bounds__(kQueueThreads) void beam_init_kernel(BeamCtrl *ctrl
     }
     if (t < n_rows) {
         seen_count[t] = 0;
-        row_done[t] = 0;
+        row_quiet[t] = 0;
     }
     if (t < n_rows * VL) {  // Queue.initialize_from_queue, queue.py:30-35
         int64_t r = t / VL;
@@ -375,7 +375,7 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
     __shared__ int n_ex_s;
     __shared__ int32_t newv[kMaxVisit];
     __shared__ int n_new_s;
-    __shared__ uint64_t tail_s;  // per-query stop: the key that ends up in the search queue's last slot
+    __shared__ int row_changed_s;  // per-query stop: some slot of the search queue's first L changed
 
     // Every global read of this workgroup is issued up front, before any of them
     // is waited for: the control words, the candidates, both queues, the popped
@@ -418,6 +418,7 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
     if (threadIdx.x == 0) {
         n_ex_s = a.excl ? a.excl_cols : 0;
         n_new_s = 0;
+        row_changed_s = 0;
     }
     __syncthreads();
     if (a.excl) {
@@ -545,7 +546,6 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
                 qi[r] = vl_key_id(k);
                 qd[r] = vl_key_dist(k);
             }
-            if (r == a.L - 1) tail_s = k;
         }
         for (int j = threadIdx.x; j < n_s; j += blockDim.x) {
             uint64_t k = cc[j];
@@ -555,21 +555,29 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
                 qd[r] = vl_key_dist(k);
                 diff = true;  // a new id inside the first L slots: the row changed (queue.py:57-59)
             }
-            if (r == a.L - 1) tail_s = k;
         }
     }
     int *flag = &c->changed[(t / a.readahead) & 63];  // every writer stores the same 1: no atomic needed
-    if (!a.row_done && checking && __ballot(diff) && lane == 0) {
+    if (a.row_quiet) {
+        // Per-query stop: a row is finished after `readahead` iterations in a row that left its first L
+        // slots as they were, or when the visited list has no free column (no pop yields a real id from
+        // then on); a row that is not finished at a checking iteration keeps the loop going.
+        if (diff) row_changed_s = 1;  // every writer stores the same 1
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int quiet = row_changed_s ? 0 : a.row_quiet[row] + 1;
+            if (seen_full) quiet = a.readahead;
+            a.row_quiet[row] = quiet;
+            if (checking && quiet < a.readahead &&
+                __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
+                __hip_atomic_store(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    } else if (checking && __ballot(diff) && lane == 0) {
         if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
             __hip_atomic_store(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (seen_full) {
-        // no pop yields a real id from now on: with the per-query stop the row is finished
-        if (a.row_done && threadIdx.x == 0) a.row_done[row] = 1;
-        return;
-    }
+    if (seen_full) return;
     __syncthreads();  // cc is reused below
-    const uint64_t tail = n_s ? tail_s : ws;
 
     // ---- visit_queue.insert(candidates, exclude=seen) : ann.py:85-88 --------------------
     auto keep_visit = [&](int i) -> bool {
@@ -601,17 +609,6 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
         vi[r] = VL_MAXINT;
         vd[r] = VL_MAXFLOAT;
     }
-    if (a.row_done && threadIdx.x == 0) {
-        // Per-query stop: the row is finished when the best node it has not visited yet is farther than the
-        // last slot of its search queue (or nothing is left to visit); otherwise it keeps the loop going.
-        uint64_t head = kPadKey;
-        if (nva > 0) head = va[0];
-        if (n_v > 0 && cc[0] < head) head = cc[0];
-        const bool done = head == kPadKey || vl_key_id(head) == VL_MAXINT || head > tail;
-        if (done) a.row_done[row] = 1;
-        else if (checking && __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
-            __hip_atomic_store(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
 }
 
 template <int THREADS>
@@ -635,6 +632,7 @@ struct StepArgs {
     uint64_t *memo;
     int memo_shift;
     int count_evals;
+    int l2;  // 0: cosine distance, 1: squared L2
 };
 
 template <int CPL, int LPR, int U, bool GENERIC, int THREADS>
@@ -646,7 +644,7 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
     const int gate = beam_gate(c, t, a.readahead, a.E, blockIdx.x == 0 && threadIdx.x == 0);
     if (gate == 2) return;
     const int64_t row = blockIdx.x;
-    if (gate == 1 || (a.row_done && a.row_done[row])) {
+    if (gate == 1 || (a.row_quiet && a.row_quiet[row] >= a.readahead)) {
         // the visit queue is no longer fed (every candidate of this iteration is empty), or this row has
         // stopped on its own: nothing changes, only the running maximum is kept current
         if (threadIdx.x == 0) raise_running_max(&c->first[(t + 1) % 3], a.seen_count[row], min(a.E, a.Vt * t));
@@ -686,9 +684,9 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
         }
         if (s.count_evals) n_fetched += __popcll(__ballot(ok));
         if constexpr (GENERIC)
-            wave_distances_generic(q_row, s.vectors, s.dim, s.nchunks, id, ok, ld + c0, memo_row, s.memo_shift);
+            wave_distances_generic(q_row, s.vectors, s.dim, s.nchunks, id, ok, ld + c0, memo_row, s.memo_shift, s.l2 != 0);
         else
-            wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, id, ok, ld + c0, memo_row, s.memo_shift);
+            wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, id, ok, ld + c0, memo_row, s.memo_shift, s.l2 != 0);
     }
     if (s.count_evals && lane == 0) {
         const int stripe = (int)((blockIdx.x * (THREADS / kWave) + wave) & (kBeamStripes - 1));
@@ -728,7 +726,7 @@ int launch_step_by_dim(const StepArgs &s, bool aligned, int threads, size_t smem
 
 struct BeamLayout {
     int64_t m, VL, Vt, E, head;
-    int64_t off_cand_ids, off_cand_d, off_v_ids, off_v_d, off_seen, off_seen_count, off_row_done, off_ctrl, off_memo, total;
+    int64_t off_cand_ids, off_cand_d, off_v_ids, off_v_d, off_seen, off_seen_count, off_row_quiet, off_ctrl, off_memo, total;
     int memo_slots;
 };
 
@@ -742,6 +740,7 @@ int beam_layout(const vl_beam_params *p, BeamLayout *l) {
                "configuration values must be positive");
     VL_REQUIRE(p->queue_length > 0 && p->queue_length < p->queue_capacity, "queue length must be below its capacity");
     VL_REQUIRE(p->n_vectors < (1ll << 30), "ids must stay below 2^30");
+    VL_REQUIRE(p->metric == VL_METRIC_COSINE || p->metric == VL_METRIC_L2, "unknown metric %lld", (long long)p->metric);
     VL_REQUIRE(p->n_rows <= kMaxBlocks, "a batch of %lld rows is too large for one call (limit %lld)",
                (long long)p->n_rows, (long long)kMaxBlocks);
     l->VL = p->visit_queue_factor * p->beam_size;                                      // ann.py:51
@@ -763,7 +762,7 @@ int beam_layout(const vl_beam_params *p, BeamLayout *l) {
     l->off_v_d = o; o = align256(o + p->n_rows * l->VL * 4);
     l->off_seen = o; o = align256(o + p->n_rows * l->E * 4);
     l->off_seen_count = o; o = align256(o + p->n_rows * 4);
-    l->off_row_done = o; o = align256(o + p->n_rows * 4);
+    l->off_row_quiet = o; o = align256(o + p->n_rows * 4);
     l->off_ctrl = o; o = align256(o + (int64_t)sizeof(BeamCtrl));
     // per-row cache of evaluated (id, distance) pairs: 128 slots per candidate of one iteration,
     // 1Ki..64Ki per row, the whole table at most 8 GiB (measured at 1M x 768: 16Ki -> 64Ki slots cuts the
@@ -817,7 +816,7 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
     float *v_d = (float *)(ws + l.off_v_d);
     int32_t *seen = (int32_t *)(ws + l.off_seen);
     int32_t *seen_count = (int32_t *)(ws + l.off_seen_count);
-    int32_t *row_done = (int32_t *)(ws + l.off_row_done);
+    int32_t *row_quiet = (int32_t *)(ws + l.off_row_quiet);
     BeamCtrl *ctrl = (BeamCtrl *)(ws + l.off_ctrl);
 
     {
@@ -826,7 +825,7 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
         if (n < p->n_rows) n = p->n_rows;
         hipLaunchKernelGGL(beam_init_kernel, dim3((unsigned)((n + kQueueThreads - 1) / kQueueThreads)),
                            dim3(kQueueThreads), 0, st, ctrl, p->n_rows, q_ids, q_dists, (int)p->queue_capacity,
-                           (int)l.head, v_ids, v_d, (int)l.VL, seen_count, row_done);
+                           (int)l.head, v_ids, v_d, (int)l.VL, seen_count, row_quiet);
         VL_LAUNCH_CHECK("beam_init_kernel");
     }
     uint64_t *memo = (uint64_t *)(ws + l.off_memo);
@@ -844,7 +843,7 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
     a.v_ids = v_ids; a.v_d = v_d; a.VL = (int)l.VL; a.Vt = (int)l.Vt; a.Pv = vl_next_pow2(l.VL + l.m);
     a.seen = seen; a.seen_count = seen_count; a.E = (int)l.E;
     const bool per_query = (p->flags & VL_BEAM_PER_QUERY_STOP) != 0;
-    a.row_done = per_query ? row_done : nullptr;
+    a.row_quiet = per_query ? row_quiet : nullptr;
     a.Pc = vl_next_pow2(l.m);
     if (a.Pc < 2) a.Pc = 2;
     // VL_BEAM_MERGE=sort selects the full-row-sort form of the merge step (exact for queue rows in any state)
@@ -877,6 +876,7 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
     StepArgs step;
     step.queries = queries; step.vectors = vectors; step.beams = beams; step.n_vectors = p->n_vectors;
     step.dim = (int)p->dim; step.nchunks = (int)((p->dim + 3) / 4); step.width = (int)p->width;
+    step.l2 = p->metric == VL_METRIC_L2;
     step.memo = l.memo_slots > 0 ? memo : nullptr;
     step.memo_shift = 32;
     if (step.memo) {
@@ -920,7 +920,7 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
             }
             rc = vl_launch_expand(queries, p->n_rows, vectors, p->n_vectors, p->dim, nullptr, v_ids, l.Vt, beams,
                                   p->n_vectors, p->width, l.m, cand_ids, cand_d, ctrl, (int)t, R, (int)l.E, l.VL,
-                                  prof ? 1 : 0, memo, l.memo_slots, st);
+                                  prof ? 1 : 0, memo, l.memo_slots, (int)p->metric, st);
             if (rc < 0) return rc;
             if (prof) VL_HIP(hipEventRecord(ev[3 * r + 1], st));
             if (use_sort_merge)

@@ -48,6 +48,7 @@ struct ExpandArgs {
     int m;     // candidates per row
     int cw;    // candidates per wavefront (<= 64)
     int parts; // workgroups per row
+    int l2;    // 0: cosine distance (the reference's), 1: squared L2
 };
 
 // blockIdx -> (row, part) so that all workgroups of one row, and the same rows
@@ -121,9 +122,9 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs a) {
     }
     const float *q_row = a.queries + row * a.dim;
     if constexpr (GENERIC)
-        wave_distances_generic(q_row, a.vectors, a.dim, a.nchunks, id, ok, out_d, memo_row, a.memo_shift);
+        wave_distances_generic(q_row, a.vectors, a.dim, a.nchunks, id, ok, out_d, memo_row, a.memo_shift, a.l2 != 0);
     else
-        wave_distances<CPL, LPR, U>(q_row, a.vectors, a.dim, a.nchunks, id, ok, out_d, memo_row, a.memo_shift);
+        wave_distances<CPL, LPR, U>(q_row, a.vectors, a.dim, a.nchunks, id, ok, out_d, memo_row, a.memo_shift, a.l2 != 0);
 }
 
 template <int CPL, int LPR, int U>
@@ -157,8 +158,9 @@ int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors,
                      const int32_t *beams, int64_t n_nodes, int64_t width, int64_t m,
                      int32_t *idx_out, float *dist_out, BeamCtrl *ctrl, int iter, int readahead,
                      int seen_cols, int64_t visit_stride, int count_evals, uint64_t *memo, int memo_slots,
-                     hipStream_t st) {
+                     int metric, hipStream_t st) {
     if (n_rows == 0 || m == 0) return VL_OK;
+    VL_REQUIRE(metric == VL_METRIC_COSINE || metric == VL_METRIC_L2, "unknown metric %d", metric);
     VL_REQUIRE(dim >= 1 && dim <= (1 << 24), "dim %lld out of range", (long long)dim);
     VL_REQUIRE(m <= (1 << 24), "row of %lld candidates is too wide", (long long)m);
     ExpandArgs a;
@@ -166,6 +168,7 @@ int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors,
     a.idx_out = idx_out; a.dist_out = dist_out;
     a.ctrl = ctrl; a.iter = iter; a.readahead = readahead; a.seen_cols = seen_cols;
     a.visit_stride = (int)visit_stride;
+    a.l2 = metric == VL_METRIC_L2;
     a.count_evals = ctrl ? count_evals : 0;
     a.memo = memo_slots > 0 ? memo : nullptr;
     a.memo_shift = 32;
@@ -208,14 +211,33 @@ int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors,
     return VL_OK;
 }
 
-VL_EXPORT int vl_gather_distances(const float *queries, int64_t n_rows, const float *vectors,
-                                  int64_t n_vectors, int64_t dim, const int32_t *ids,
-                                  int64_t width, float *out, void *stream) {
+VL_EXPORT int vl_gather_distances_metric(const float *queries, int64_t n_rows, const float *vectors,
+                                         int64_t n_vectors, int64_t dim, const int32_t *ids,
+                                         int64_t width, int metric, float *out, void *stream) {
     VL_REQUIRE(n_rows >= 0 && width >= 0 && n_vectors >= 0, "negative size");
     if (n_rows == 0 || width == 0) return VL_OK;
     VL_REQUIRE(queries && vectors && ids && out, "null pointer");
     return vl_launch_expand(queries, n_rows, vectors, n_vectors, dim, ids, nullptr, 0, nullptr, 0,
-                            width, width, nullptr, out, nullptr, 0, 1, 0, 0, 0, nullptr, 0, (hipStream_t)stream);
+                            width, width, nullptr, out, nullptr, 0, 1, 0, 0, 0, nullptr, 0, metric, (hipStream_t)stream);
+}
+
+VL_EXPORT int vl_gather_distances(const float *queries, int64_t n_rows, const float *vectors,
+                                  int64_t n_vectors, int64_t dim, const int32_t *ids,
+                                  int64_t width, float *out, void *stream) {
+    return vl_gather_distances_metric(queries, n_rows, vectors, n_vectors, dim, ids, width, VL_METRIC_COSINE, out, stream);
+}
+
+VL_EXPORT int vl_search_from_seeds_metric(const float *queries, int64_t n_rows, int64_t dim,
+                                          const int32_t *visit, int64_t n_visit, const int32_t *beams,
+                                          int64_t n_nodes, int64_t width, const float *vectors,
+                                          int64_t n_vectors, int metric, int32_t *idx_out, float *dist_out,
+                                          void *stream) {
+    VL_REQUIRE(n_rows >= 0 && n_visit >= 0 && width >= 0, "negative size");
+    if (n_rows == 0 || n_visit == 0 || width == 0) return VL_OK;
+    VL_REQUIRE(queries && visit && beams && vectors && idx_out && dist_out, "null pointer");
+    return vl_launch_expand(queries, n_rows, vectors, n_vectors, dim, nullptr, visit, n_visit, beams,
+                            n_nodes, width, n_visit * width, idx_out, dist_out, nullptr, 0, 1, 0, n_visit, 0, nullptr, 0,
+                            metric, (hipStream_t)stream);
 }
 
 VL_EXPORT int vl_search_from_seeds(const float *queries, int64_t n_rows, int64_t dim,
@@ -223,10 +245,6 @@ VL_EXPORT int vl_search_from_seeds(const float *queries, int64_t n_rows, int64_t
                                    int64_t n_nodes, int64_t width, const float *vectors,
                                    int64_t n_vectors, int32_t *idx_out, float *dist_out,
                                    void *stream) {
-    VL_REQUIRE(n_rows >= 0 && n_visit >= 0 && width >= 0, "negative size");
-    if (n_rows == 0 || n_visit == 0 || width == 0) return VL_OK;
-    VL_REQUIRE(queries && visit && beams && vectors && idx_out && dist_out, "null pointer");
-    return vl_launch_expand(queries, n_rows, vectors, n_vectors, dim, nullptr, visit, n_visit, beams,
-                            n_nodes, width, n_visit * width, idx_out, dist_out, nullptr, 0, 1, 0, n_visit, 0, nullptr, 0,
-                            (hipStream_t)stream);
+    return vl_search_from_seeds_metric(queries, n_rows, dim, visit, n_visit, beams, n_nodes, width, vectors, n_vectors,
+                                       VL_METRIC_COSINE, idx_out, dist_out, stream);
 }

@@ -12,6 +12,11 @@ __device__ __forceinline__ float clamp_distance(float cos_theta) {
     return r;
 }
 
+// The folded sum as a distance.  Cosine (the reference's only metric, kernels.py:85-114): the sum is
+// the dot product.  Squared L2 (an addition): the sum already is sum_j (a_j - b_j)^2, taken in the
+// same chunk / lane / fold order with one subtraction and one fused multiply-add per element.
+__device__ __forceinline__ float finish_distance(float sum, bool l2) { return l2 ? sum : clamp_distance(sum); }
+
 // Per-row cache of distances already evaluated in this search: slot = hash(id),
 // entry = (distance bits << 32) | id.  Several wavefronts read and write a row's
 // table concurrently, so an entry is always moved as ONE relaxed 64-bit atomic
@@ -63,7 +68,7 @@ __device__ __forceinline__ void wave_distances(const float *__restrict__ q_row,
                                                const float *__restrict__ vectors, int dim,
                                                int nchunks, int32_t my_id, bool ok,
                                                float *__restrict__ out_d, uint64_t *memo_row,
-                                               int memo_shift) {
+                                               int memo_shift, bool l2 = false) {
     constexpr int G = kWave / LPR;
     const int lane = threadIdx.x & (kWave - 1);
     const int grp = lane / LPR;
@@ -119,16 +124,28 @@ __device__ __forceinline__ void wave_distances(const float *__restrict__ q_row,
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             float acc = 0.0f;
+            if (l2) {  // uniform over the launch
 #pragma unroll
-            for (int i = 0; i < CPL; ++i) {
-                acc = __builtin_fmaf(r[u][i].x, q[i].x, acc);
-                acc = __builtin_fmaf(r[u][i].y, q[i].y, acc);
-                acc = __builtin_fmaf(r[u][i].z, q[i].z, acc);
-                acc = __builtin_fmaf(r[u][i].w, q[i].w, acc);
+                for (int i = 0; i < CPL; ++i) {
+                    const float dx = r[u][i].x - q[i].x, dy = r[u][i].y - q[i].y;
+                    const float dz = r[u][i].z - q[i].z, dw = r[u][i].w - q[i].w;
+                    acc = __builtin_fmaf(dx, dx, acc);
+                    acc = __builtin_fmaf(dy, dy, acc);
+                    acc = __builtin_fmaf(dz, dz, acc);
+                    acc = __builtin_fmaf(dw, dw, acc);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < CPL; ++i) {
+                    acc = __builtin_fmaf(r[u][i].x, q[i].x, acc);
+                    acc = __builtin_fmaf(r[u][i].y, q[i].y, acc);
+                    acc = __builtin_fmaf(r[u][i].z, q[i].z, acc);
+                    acc = __builtin_fmaf(r[u][i].w, q[i].w, acc);
+                }
             }
             acc = fold_group<LPR>(acc);
             if (lig == 0 && mysrc[u] >= 0) {
-                float d = clamp_distance(acc);
+                float d = finish_distance(acc, l2);
                 out_d[mysrc[u]] = d;
                 if (memo_row) memo_store(memo_row, memo_shift, ids[u], d);
             }
@@ -141,7 +158,7 @@ __device__ __forceinline__ void wave_distances_generic(const float *__restrict__
                                                        const float *__restrict__ vectors, int dim,
                                                        int nchunks, int32_t my_id, bool ok,
                                                        float *__restrict__ out_d, uint64_t *memo_row,
-                                                       int memo_shift) {
+                                                       int memo_shift, bool l2 = false) {
     const int lane = threadIdx.x & (kWave - 1);
     uint64_t mask = __ballot(ok);
     while (mask) {
@@ -154,12 +171,15 @@ __device__ __forceinline__ void wave_distances_generic(const float *__restrict__
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 int i = 4 * c + j;
-                if (i < dim) acc = __builtin_fmaf(row[i], q_row[i], acc);
+                if (i < dim) {
+                    const float x = l2 ? row[i] - q_row[i] : row[i];
+                    acc = __builtin_fmaf(x, l2 ? x : q_row[i], acc);
+                }
             }
         }
         acc = fold_group<kWave>(acc);
         if (lane == 0) {
-            float d = clamp_distance(acc);
+            float d = finish_distance(acc, l2);
             out_d[s] = d;
             if (memo_row) memo_store(memo_row, memo_shift, id, d);
         }

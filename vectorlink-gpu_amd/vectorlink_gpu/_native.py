@@ -20,14 +20,26 @@ class BeamParams(C.Structure):
     _fields_ = [(n, C.c_int64) for n in (
         "n_rows", "dim", "n_vectors", "width", "queue_capacity", "queue_length", "beam_size",
         "parallel_visit_count", "visit_queue_factor", "exclude_factor", "speculative_readahead", "excl_cols",
-        "flags")]
+        "flags", "metric")]
+
+
+METRICS = {"cosine": 0, "l2": 1}  # include/vlgpu.h: VL_METRIC_COSINE, VL_METRIC_L2
+
+
+def metric_code(name: str) -> int:
+    if name not in METRICS:
+        raise ValueError(f"unknown metric {name!r}: expected one of {sorted(METRICS)}")
+    return METRICS[name]
 
 
 _SIGNATURES = {
     "vl_last_error": (C.c_char_p, []),
     "vl_version": (C.c_int, []),
     "vl_gather_distances": (C.c_int, [_ptr, _i64, _ptr, _i64, _i64, _ptr, _i64, _ptr, _ptr]),
+    "vl_gather_distances_metric": (C.c_int, [_ptr, _i64, _ptr, _i64, _i64, _ptr, _i64, C.c_int, _ptr, _ptr]),
     "vl_search_from_seeds": (C.c_int, [_ptr, _i64, _i64, _ptr, _i64, _ptr, _i64, _i64, _ptr, _i64, _ptr, _ptr, _ptr]),
+    "vl_search_from_seeds_metric": (C.c_int, [_ptr, _i64, _i64, _ptr, _i64, _ptr, _i64, _i64, _ptr, _i64, C.c_int, _ptr,
+                                              _ptr, _ptr]),
     "vl_circulants": (C.c_int, [_ptr, _i64, _i64, _i64, _ptr, _i64, _ptr]),
     "vl_dedup_ids": (C.c_int, [_ptr, _i64, _i64, _ptr]),
     "vl_dedup_pairs": (C.c_int, [_ptr, _ptr, _i64, _i64, _ptr]),

@@ -33,7 +33,7 @@ def _beam_params(batch: int, dim: int, n_vectors: int, width: int, queue: Queue,
         queue_length=queue.length, beam_size=config["beam_size"],
         parallel_visit_count=config["parallel_visit_count"], visit_queue_factor=config["visit_queue_factor"],
         exclude_factor=config["exclude_factor"], speculative_readahead=config["speculative_readahead"],
-        excl_cols=excl_cols, flags=flags)
+        excl_cols=excl_cols, flags=flags, metric=nv.metric_code(config.get("metric", "cosine")))
 
 
 class _Workspace:
@@ -92,7 +92,7 @@ def closest_vectors_stepwise(query_vecs: Tensor, search_queue: Queue, vectors: T
         checking_output = (count % config["speculative_readahead"]) == 0
         neighbors_to_visit = visit_queue.pop_n_ids(config["parallel_visit_count"])
         (indexes_of_comparisons, distances_of_comparisons) = search_from_seeds(
-            query_vecs, neighbors_to_visit, beams, vectors)
+            query_vecs, neighbors_to_visit, beams, vectors, config.get("metric", "cosine"))
         did_something = search_queue.insert(indexes_of_comparisons, distances_of_comparisons, exclude=exclude,
                                             output_update=checking_output)
         if seen is not None:
@@ -175,7 +175,7 @@ class GraphBuild:
         if initial is None:
             neighbor_primes = primes(self.queue_length, device)
             self.beams = generate_circulant_beams(self.num_vecs, neighbor_primes)
-            self.beam_distances = calculate_distances(vectors, self.beams)  # of the circulant graph
+            self.beam_distances = calculate_distances(vectors, self.beams, metric=config.get("metric", "cosine"))
         else:
             (self.beams, self.beam_distances) = initial
             assert self.beams.size() == (self.num_vecs, self.queue_length) == self.beam_distances.size()
@@ -237,7 +237,7 @@ class GraphBuild:
         if self.config["prune"] == "rank":
             # addition: cut the full-width table to beam_size by detour count and merge reverse edges
             ids = optimize_graph(self.beams, self.beam_size)
-            return (ids, gather_distances(self.vectors, self.vectors, ids))
+            return (ids, gather_distances(self.vectors, self.vectors, ids, metric=self.config.get("metric", "cosine")))
         out_distances = self.beam_distances if self.stale else self.distances  # ann.py:190-193
         return (self.beams.narrow_copy(1, 0, self.beam_size), out_distances.narrow_copy(1, 0, self.beam_size))
 
@@ -263,19 +263,20 @@ def initial_queue(vectors: Tensor, config: Dict) -> Queue:
     queue = Queue(batch_size, queue_size, queue_size + extra_capacity, device=vectors.device)
     p = primes(queue_size, vectors.device)
     initial_queue_indices = generate_circulant_beams(batch_size, p)
-    d = calculate_distances(vectors, initial_queue_indices)
+    d = calculate_distances(vectors, initial_queue_indices, metric=config.get("metric", "cosine"))
     queue.insert(initial_queue_indices, d)
     return queue
 
 
-def query_cosine_distances(query_vectors: Tensor, vectors: Tensor, ids: Tensor) -> Tensor:
+def query_cosine_distances(query_vectors: Tensor, vectors: Tensor, ids: Tensor, metric: str = "cosine") -> Tensor:
     """d[b, j] = clamp((1 - <query[b], vectors[ids[b, j]]>) / 2, 0, 1).
 
     The reference's version (ann.py:211-214) multiplies [B, D] by a gathered
     [B, Q, D] tensor, which only broadcasts for one query, and leaves out the
     clamp; this one evaluates the seeds with the kernel every other distance
-    uses, so a seed found again during the search carries identical bits."""
-    return gather_distances(query_vectors, vectors, ids)
+    uses, so a seed found again during the search carries identical bits.
+    metric="l2" (an addition) gives squared Euclidean distances instead."""
+    return gather_distances(query_vectors, vectors, ids, metric=metric)
 
 
 def initial_search_queue(vectors: Tensor, query_vectors: Tensor, config: Dict,
@@ -289,7 +290,7 @@ def initial_search_queue(vectors: Tensor, query_vectors: Tensor, config: Dict,
     p = primes(queue_size, vectors.device)
     (vector_count, _) = vectors.size()
     initial_queue_indices = generate_queue_circulants(batch_size, vector_count, p)
-    d = query_cosine_distances(query_vectors, vectors, initial_queue_indices)
+    d = query_cosine_distances(query_vectors, vectors, initial_queue_indices, config.get("metric", "cosine"))
     queue.insert(initial_queue_indices, d)
     return queue
 
@@ -319,7 +320,7 @@ def dense_search_queue(vectors: Tensor, query_vectors: Tensor, config: Dict, ent
     k = min(DENSE_SEEDS, entry_ids.size(0), queue_size)
     (local, _) = knn_exact(query_vectors, entry_vectors, k)
     seeds = entry_ids[local.long()].contiguous()
-    d = query_cosine_distances(query_vectors, vectors, seeds)
+    d = query_cosine_distances(query_vectors, vectors, seeds, config.get("metric", "cosine"))
     queue.insert(seeds, d)
     return queue
 
@@ -399,14 +400,20 @@ class ANN:
         seeding: str = "circulant",
         entry_points: int = 32_768,
         keep_queues: bool = False,
+        metric: str = "cosine",
     ):
         """seeding / entry_points are additions: "circulant" seeds searches as the
         reference does; "dense" seeds them from the nearest of `entry_points`
         evenly spread vectors (see dense_search_queue).  prune also accepts
         "rank": no pruning between loops, and the final cut from the build queue
         width to beam_size is done by detour count with reverse edges merged in
-        (kernels.optimize_graph) instead of keeping the first beam_size columns."""
+        (kernels.optimize_graph) instead of keeping the first beam_size columns.
+        metric is an addition too: "cosine" is the reference's distance; "l2" builds
+        and searches by squared Euclidean distance (rows need not be unit length;
+        the dense seeding and recall_at_k tiles are cosine only and refuse it)."""
         assert prune in (True, False, "rank")
+        nv.metric_code(metric)
+        assert not (metric == "l2" and seeding == "dense"), "dense seeding is cosine only"
         assert vectors.dim() == 2 and vectors.dtype == torch.float32
         assert seeding in ("circulant", "dense")
         self.seeding = seeding
@@ -426,6 +433,8 @@ class ANN:
             "recall_search_queue_factor": recall_search_queue_factor,
             "speculative_readahead": speculative_readahead,
         }
+        if metric != "cosine":
+            self.configuration["metric"] = metric
         if not vectors.is_cuda:
             vectors = vectors.to(DEVICE)
         self.vectors = vectors.contiguous()
@@ -433,7 +442,7 @@ class ANN:
         if beams is not None:
             self.beams = beams.to(self.vectors.device).contiguous()
             if distances is None:
-                self.distances = calculate_distances(self.vectors, self.beams)
+                self.distances = calculate_distances(self.vectors, self.beams, metric=metric)
             else:
                 self.distances = distances.to(self.vectors.device).contiguous()
         else:
@@ -528,9 +537,9 @@ class ANN:
         queue_size overrides the configured search-queue length, seeding the
         instance's seeding mode.  stop="batch" is the reference's loop (every row
         expands until no row of the batch changed at a progress check);
-        stop="per_query" ends each row on its own once its best unvisited node is
-        farther than the last slot of its queue - faster for large batches, not
-        the reference's result."""
+        stop="per_query" finishes each row on its own after speculative_readahead
+        iterations in a row that left its queue unchanged - faster for large
+        batches, not the reference's result."""
         assert stop in ("batch", "per_query")
         assert query.dim() == 2 and query.dtype == torch.float32
         if not query.is_cuda:
@@ -538,6 +547,8 @@ class ANN:
         query = query.contiguous()
         seeding = seeding or self.seeding
         assert seeding in ("circulant", "dense")
+        if seeding == "dense" and self.configuration.get("metric", "cosine") != "cosine":
+            raise ValueError("dense seeding ranks entry points by cosine distance; use circulant seeds with metric='l2'")
         if seeding == "dense":
             (entry_ids, entry_vectors) = self._entry_tables()
             search_queue = dense_search_queue(self.vectors, query, self.configuration, entry_ids, entry_vectors,
@@ -553,6 +564,8 @@ class ANN:
         """Share of the exact k nearest neighbours (brute force on MFMA tiles)
         that search() returns in its first k slots.  Not in the reference,
         whose recall() is self-recall@1."""
+        if self.configuration.get("metric", "cosine") != "cosine":
+            raise ValueError("the exact-kNN tiles are cosine only")
         if not query.is_cuda:
             query = query.to(self.vectors.device)
         query = query.contiguous()

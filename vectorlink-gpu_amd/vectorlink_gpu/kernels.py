@@ -21,8 +21,10 @@ def _check_f32(t: Tensor, name: str):
     assert t.is_contiguous(), f"{name} must be contiguous"
 
 
-def gather_distances(queries: Tensor, vectors: Tensor, ids: Tensor, out: Optional[Tensor] = None) -> Tensor:
-    """out[r, j] = cosine distance of queries[r] and vectors[ids[r, j]] (MAXFLOAT for MAXINT ids)."""
+def gather_distances(queries: Tensor, vectors: Tensor, ids: Tensor, out: Optional[Tensor] = None,
+                     metric: str = "cosine") -> Tensor:
+    """out[r, j] = distance of queries[r] and vectors[ids[r, j]] (MAXFLOAT for MAXINT ids): the reference's
+    cosine distance, or with metric="l2" (an addition) the squared Euclidean distance."""
     _check_f32(queries, "queries")
     _check_f32(vectors, "vectors")
     _check_ids(ids, "ids")
@@ -34,24 +36,26 @@ def gather_distances(queries: Tensor, vectors: Tensor, ids: Tensor, out: Optiona
     else:
         _check_f32(out, "out")
         assert out.size() == ids.size()
-    nv.check(nv.lib().vl_gather_distances(nv.ptr(queries), rows, nv.ptr(vectors), vectors.size(0), vectors.size(1),
-                                          nv.ptr(ids), width, nv.ptr(out), nv.stream()))
+    nv.check(nv.lib().vl_gather_distances_metric(nv.ptr(queries), rows, nv.ptr(vectors), vectors.size(0),
+                                                 vectors.size(1), nv.ptr(ids), width, nv.metric_code(metric),
+                                                 nv.ptr(out), nv.stream()))
     return out
 
 
 @log_time
-def calculate_distances(vectors: Tensor, beams: Tensor, distances_out: Optional[Tensor] = None) -> Tensor:
+def calculate_distances(vectors: Tensor, beams: Tensor, distances_out: Optional[Tensor] = None,
+                        metric: str = "cosine") -> Tensor:
     """reference kernels.py:174-201"""
     _check_f32(vectors, "vectors")
     _check_ids(beams, "beams")
     (vector_count, _) = vectors.size()
     (batches, _) = beams.size()
     assert batches == vector_count  # kernels.py:186
-    return gather_distances(vectors, vectors, beams, distances_out)
+    return gather_distances(vectors, vectors, beams, distances_out, metric)
 
 
 def search_from_seeds(query_vecs: Tensor, neighbors_to_visit: Tensor, beams: Tensor,
-                      vectors: Tensor) -> Tuple[Tensor, Tensor]:
+                      vectors: Tensor, metric: str = "cosine") -> Tuple[Tensor, Tensor]:
     """reference kernels.py:260-311"""
     _check_f32(query_vecs, "query_vecs")
     _check_ids(neighbors_to_visit, "neighbors_to_visit")
@@ -64,9 +68,10 @@ def search_from_seeds(query_vecs: Tensor, neighbors_to_visit: Tensor, beams: Ten
     assert query_vecs.size(0) == batch_size and query_vecs.size(1) == dim
     index_out = torch.empty((batch_size, visit_length * beam_size), dtype=torch.int32, device=vectors.device)
     distance_out = torch.empty((batch_size, visit_length * beam_size), dtype=torch.float32, device=vectors.device)
-    nv.check(nv.lib().vl_search_from_seeds(nv.ptr(query_vecs), batch_size, dim, nv.ptr(neighbors_to_visit),
-                                           visit_length, nv.ptr(beams), node_count, beam_size, nv.ptr(vectors),
-                                           vector_count, nv.ptr(index_out), nv.ptr(distance_out), nv.stream()))
+    nv.check(nv.lib().vl_search_from_seeds_metric(nv.ptr(query_vecs), batch_size, dim, nv.ptr(neighbors_to_visit),
+                                                  visit_length, nv.ptr(beams), node_count, beam_size, nv.ptr(vectors),
+                                                  vector_count, nv.metric_code(metric), nv.ptr(index_out),
+                                                  nv.ptr(distance_out), nv.stream()))
     return (index_out, distance_out)
 
 
