@@ -98,3 +98,15 @@ def test_cpu_tensors_are_refused():
     q = Queue(2, 2, 6, device="cpu")
     with pytest.raises(RuntimeError):
         q.insert(torch.zeros((2, 2), dtype=torch.int32), torch.zeros((2, 2), dtype=torch.float32))
+
+
+def test_library_is_not_older_than_its_sources():
+    """The built library travels with the tree; one that predates an edit of its sources would be
+    tested in their place."""
+    from vectorlink_gpu import _native
+
+    built = os.path.getmtime(_native.LIB_PATH)
+    csrc = os.path.join(ROOT, "vectorlink-gpu_amd", "csrc")
+    sources = [os.path.join(csrc, f) for f in os.listdir(csrc)] + [HEADER]
+    stale = [os.path.basename(s) for s in sources if os.path.getmtime(s) > built]
+    assert not stale, f"rebuild libvlgpu.so (python vectorlink-gpu_amd/build.py): newer sources {stale}"
