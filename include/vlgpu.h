@@ -214,6 +214,34 @@ int64_t vl_closest_vectors(const vl_beam_params *p,
                            void *workspace, int64_t workspace_bytes,
                            void *stream);
 
+/* vl_closest_vectors for callers that cannot allocate or wait: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has
+ * no counterpart in the reference.  Differences from vl_closest_vectors:
+ *  - no workspace argument: the loop's scratch memory (control block, visit
+ *    queues, visited lists; the fused step only, without the per-row distance
+ *    cache) is a static device array of VL_NOALLOC_SCRATCH_BYTES inside the
+ *    library, which every GPU the library runs on holds until the process
+ *    ends.  A batch that needs more (about 8 * visit queue length + 4 * visited
+ *    list length bytes per row) is refused with VL_ERR_ARG; nothing is
+ *    allocated or freed, here or in anything this call uses;
+ *  - no host round trips: exactly `iterations` launches are enqueued and the
+ *    call returns 0 at once.  When a progress check finds the batch quiet the
+ *    remaining launches do nothing, so with iterations >= the count
+ *    vl_closest_vectors would return the queues end up bit-identical to its;
+ *  - status_out (device, 2 x int32) receives [0] = 1 if the loop ended within
+ *    `iterations` (else 0: the queues hold an unfinished search) and [1] = the
+ *    number of iterations that ran.
+ * All calls on one GPU share that GPU's array: calls that overlap on one GPU
+ * (two streams, two threads) race; serialise them. */
+#define VL_NOALLOC_SCRATCH_BYTES (32 << 20)
+int vl_closest_vectors_noalloc(const vl_beam_params *p,
+                               const float *queries, const float *vectors,
+                               const int32_t *beams,
+                               int32_t *q_ids, float *q_dists,
+                               const int32_t *exclude,
+                               int64_t iterations, int32_t *status_out,
+                               void *stream);
+
 /* Per-kernel timing of vl_closest_vectors (no counterpart in the reference,
  * whose log.py:7-17 times whole calls): with enable != 0 every expand / merge
  * launch is bracketed by HIP events on the caller's stream.  out (8 doubles,

@@ -114,7 +114,7 @@ __global__ __launch_bounds__(kQueueThreads) void beam_init_kernel(BeamCtrl *ctrl
     int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t == 0) {
         ctrl->stop = 0;
-        ctrl->reserved = 0;
+        ctrl->ended_after = 0;
         ctrl->first[0] = ctrl->first[1] = ctrl->first[2] = 0;
     }
     if (t < 64) ctrl->changed[t] = 0;
@@ -732,7 +732,9 @@ struct BeamLayout {
 
 inline int64_t align256(int64_t x) { return (x + 255) & ~255ll; }
 
-int beam_layout(const vl_beam_params *p, BeamLayout *l) {
+// lean: the layout of the entry point that allocates nothing - the fused step keeps its candidates in LDS
+// and runs without the distance cache, so neither gets room.
+int beam_layout(const vl_beam_params *p, BeamLayout *l, bool lean = false) {
     VL_REQUIRE(p, "null params");
     VL_REQUIRE(p->n_rows >= 0 && p->dim > 0 && p->n_vectors > 0 && p->width > 0, "bad sizes");
     VL_REQUIRE(p->beam_size > 0 && p->parallel_visit_count > 0 && p->visit_queue_factor > 0 &&
@@ -756,8 +758,8 @@ int beam_layout(const vl_beam_params *p, BeamLayout *l) {
                "queue rows above %d slots are not supported", kMaxRowSlots);
     VL_REQUIRE(p->excl_cols >= 0 && p->excl_cols <= 1024, "exclusion rows above 1024 ids are not supported here");
     int64_t o = 0;
-    l->off_cand_ids = o; o = align256(o + p->n_rows * l->m * 4);
-    l->off_cand_d = o; o = align256(o + p->n_rows * l->m * 4);
+    l->off_cand_ids = o; o = align256(o + (lean ? 0 : p->n_rows * l->m * 4));
+    l->off_cand_d = o; o = align256(o + (lean ? 0 : p->n_rows * l->m * 4));
     l->off_v_ids = o; o = align256(o + p->n_rows * l->VL * 4);
     l->off_v_d = o; o = align256(o + p->n_rows * l->VL * 4);
     l->off_seen = o; o = align256(o + p->n_rows * l->E * 4);
@@ -776,6 +778,7 @@ int beam_layout(const vl_beam_params *p, BeamLayout *l) {
     if (slots > 65536) slots = 65536;
     while (slots > 1024 && p->n_rows * (int64_t)slots * 8 > (8ll << 30)) slots >>= 1;
     if (memo_env >= 0) slots = memo_env;
+    if (lean) slots = 0;
     l->memo_slots = slots;
     l->off_memo = o; o = align256(o + p->n_rows * (int64_t)slots * 8);
     l->total = o;
@@ -790,14 +793,35 @@ VL_EXPORT int64_t vl_beam_workspace_bytes(const vl_beam_params *p) {
     return rc < 0 ? rc : l.total;
 }
 
-VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queries, const float *vectors,
-                                     const int32_t *beams, int32_t *q_ids, float *q_dists,
-                                     const int32_t *exclude, void *workspace, int64_t workspace_bytes,
-                                     void *stream) {
-    BeamLayout l;
-    int rc = beam_layout(p, &l);
-    if (rc < 0) return rc;
-    if (p->n_rows == 0) return 0;
+namespace {
+
+__global__ void beam_empty_status_kernel(int32_t *status) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        status[0] = 1;
+        status[1] = 0;
+    }
+}
+
+__global__ void beam_status_kernel(const BeamCtrl *c, int iterations, int R, int32_t *status) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    int ended = c->stop, t = c->ended_after;
+    if (!ended && iterations % R == 0 && c->changed[(iterations / R) & 63] == 0) {
+        ended = 1;  // the last launch was a checking iteration that found every row quiet
+        t = iterations;
+    }
+    status[0] = ended;
+    status[1] = ended ? t : iterations;
+}
+
+// The loop itself.  fixed_iterations == 0: run until a progress check finds the batch quiet, reading the
+// flag on the host every speculative_readahead iterations; returns the iteration count.  fixed_iterations
+// > 0: enqueue exactly that many iterations and return 0 without ever waiting for the device - once a
+// check finds the batch quiet the remaining launches do nothing (beam_gate) - then one small kernel writes
+// status_out[0] = 1 if the loop ended within them (else 0) and status_out[1] = the iteration count.
+int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *queries, const float *vectors,
+                  const int32_t *beams, int32_t *q_ids, float *q_dists, const int32_t *exclude, void *workspace,
+                  int64_t workspace_bytes, int64_t fixed_iterations, int32_t *status_out, void *stream) {
+    int rc;
     VL_REQUIRE(queries && vectors && beams && q_ids && q_dists && workspace, "null pointer");
     VL_REQUIRE(((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
     if (workspace_bytes < l.total) {
@@ -886,6 +910,19 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
         step.memo_shift = 32 - lg;
     }
     const int R = (int)p->speculative_readahead;
+    if (fixed_iterations > 0) {
+        VL_REQUIRE(use_fused, "a fixed number of iterations is only built for the fused step");
+        for (int64_t t = 1; t <= fixed_iterations; ++t) {
+            a.iter = (int)t;
+            step.m = a;
+            step.count_evals = 0;
+            rc = launch_step_by_dim(step, aligned, merge_threads == 128 ? 128 : 256, smem, st);
+            if (rc < 0) return rc;
+        }
+        hipLaunchKernelGGL(beam_status_kernel, dim3(1), dim3(64), 0, st, ctrl, (int)fixed_iterations, R, status_out);
+        VL_LAUNCH_CHECK("beam_status_kernel");
+        return 0;
+    }
     bool prof;
     {
         std::lock_guard<std::mutex> hold(g_prof_mutex);
@@ -974,6 +1011,78 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
         g_prof.iterations += t;
     }
     return t;
+}
+
+}  // namespace
+
+VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queries, const float *vectors,
+                                     const int32_t *beams, int32_t *q_ids, float *q_dists,
+                                     const int32_t *exclude, void *workspace, int64_t workspace_bytes,
+                                     void *stream) {
+    BeamLayout l;
+    int rc = beam_layout(p, &l);
+    if (rc < 0) return rc;
+    if (p->n_rows == 0) return 0;
+    return beam_loop(p, l, queries, vectors, beams, q_ids, q_dists, exclude, workspace, workspace_bytes, 0, nullptr,
+                     stream);
+}
+
+// ---- the entry point that allocates nothing -------------------------------------------
+// Its scratch memory is this array, part of the loaded code object: every GPU the library runs on holds
+// its own copy until the process ends.  In host code the array's name is only a handle; the address the
+// kernels are given comes from hipGetSymbolAddress, looked up once per device with that device current.
+namespace {
+
+static __device__ __align__(256) unsigned char scratch[VL_NOALLOC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+int scratch_of_current_device(void **out) {
+    int dev = -1;
+    VL_HIP(hipGetDevice(&dev));
+    VL_REQUIRE(dev >= 0 && dev < kMaxDevices, "device index %d is out of range", dev);
+    std::lock_guard<std::mutex> hold(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        VL_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        VL_REQUIRE(ptr != nullptr, "no device address for the static scratch array");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return VL_OK;
+}
+
+}  // namespace
+
+VL_EXPORT int vl_closest_vectors_noalloc(const vl_beam_params *p, const float *queries, const float *vectors,
+                                         const int32_t *beams, int32_t *q_ids, float *q_dists,
+                                         const int32_t *exclude, int64_t iterations, int32_t *status_out,
+                                         void *stream) {
+    BeamLayout l;
+    int rc = beam_layout(p, &l, true);
+    if (rc < 0) return rc;
+    VL_REQUIRE(iterations >= 1 && iterations <= 65536, "iterations must be between 1 and 65536");
+    VL_REQUIRE(status_out, "null pointer");
+    VL_REQUIRE((p->flags & (VL_BEAM_TWO_LAUNCHES | VL_BEAM_SORT_MERGE)) == 0,
+               "only the fused step runs without a caller's workspace");
+    VL_REQUIRE(l.total <= (int64_t)VL_NOALLOC_SCRATCH_BYTES,
+               "this batch needs %lld bytes of scratch memory, the static array holds %lld: use fewer rows per call "
+               "(about %lld bytes per row) or vl_closest_vectors with a workspace",
+               (long long)l.total, (long long)VL_NOALLOC_SCRATCH_BYTES,
+               (long long)(l.VL * 8 + l.E * 4 + 8));
+    void *ptr = nullptr;
+    rc = scratch_of_current_device(&ptr);
+    if (rc < 0) return rc;
+    if (p->n_rows == 0) {
+        // nothing to search: the loop ended after no iteration
+        hipLaunchKernelGGL(beam_empty_status_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, status_out);
+        VL_LAUNCH_CHECK("beam_empty_status_kernel");
+        return VL_OK;
+    }
+    return (int)beam_loop(p, l, queries, vectors, beams, q_ids, q_dists, exclude, ptr, VL_NOALLOC_SCRATCH_BYTES,
+                          iterations, status_out, stream);
 }
 
 // Profiling switch for vl_closest_vectors: when enabled every expand / merge

@@ -15,7 +15,7 @@ constexpr int kBeamStripes = 1024;
 
 struct BeamCtrl {
     int stop;
-    int reserved;
+    int ended_after;  // iterations run when stop was set (for callers that enqueue a fixed number of launches)
     int first[3];
     int changed[64];
     // profiling only, striped by workgroup so that the atomic adds do not queue up on one address:
@@ -33,7 +33,10 @@ struct BeamCtrl {
 __device__ inline int beam_gate(BeamCtrl *c, int t, int R, int E, bool writer) {
     int stop = c->stop;
     const bool after_check = t > 1 && ((t - 1) % R) == 0;
-    if (!stop && after_check && c->changed[((t - 1) / R) & 63] == 0) stop = 1;
+    if (!stop && after_check && c->changed[((t - 1) / R) & 63] == 0) {
+        stop = 1;
+        if (writer) c->ended_after = t - 1;  // the loop ran t - 1 iterations
+    }
     if (stop) {
         if (writer) c->stop = 1;
         return 2;

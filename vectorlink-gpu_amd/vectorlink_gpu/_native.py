@@ -53,6 +53,7 @@ _SIGNATURES = {
     "vl_seen_add": (C.c_int, [_ptr, _i64, _i64, _ptr, _i64, _ptr, C.POINTER(C.c_int), _ptr]),
     "vl_beam_workspace_bytes": (C.c_int64, [C.POINTER(BeamParams)]),
     "vl_closest_vectors": (C.c_int64, [C.POINTER(BeamParams), _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr]),
+    "vl_closest_vectors_noalloc": (C.c_int, [C.POINTER(BeamParams), _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr]),
     "vl_beam_profile": (C.c_int, [C.c_int, C.c_int, C.POINTER(C.c_double)]),
     "vl_optimize_graph_workspace_bytes": (C.c_int64, [_i64, _i64, _i64]),
     "vl_optimize_graph": (C.c_int, [_ptr, _i64, _i64, _i64, _ptr, _ptr, _i64, _ptr]),
