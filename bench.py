@@ -94,6 +94,21 @@ def measured_copy_gbs(torch, dev):
     return 2.0 * (1 << 30) / (best / 1e3) / 1e9
 
 
+class Phases:
+    """Beam-search launches per phase of this run, in order, so that a profiler's list of
+    beam_step_kernel dispatches can be cut into the same phases."""
+
+    def __init__(self):
+        from vectorlink_gpu import log as vl_log
+
+        self.log, self.rows, self.last = vl_log, [], vl_log.BEAM_ITERATIONS
+
+    def mark(self, name):
+        now = self.log.BEAM_ITERATIONS
+        self.rows.append(dict(phase=name, beam_step_launches=now - self.last))
+        self.last = now
+
+
 def recall_at(found, truth):
     hits = (found.unsqueeze(2) == truth.unsqueeze(1)).any(dim=2).sum().item()
     return hits / truth.numel()
@@ -237,6 +252,7 @@ def main():
     qdev = queries.to(dev)
     torch.cuda.synchronize()
 
+    phases = Phases()
     # warm-up: a small separate build (kernels loaded, allocator primed)
     if args.warmup > 0:
         wb = GraphBuild(vectors[:50_000].contiguous(), cfg)
@@ -245,6 +261,7 @@ def main():
                 break
         torch.cuda.synchronize()
         del wb
+    phases.mark("warm-up")
 
     copy_gbs = measured_copy_gbs(torch, dev)
     log(f"[bench] 1 GiB device copy: {copy_gbs:.0f} GB/s")
@@ -259,13 +276,18 @@ def main():
     done = 0
     t_first_k = None
     t_said = t_start
+    in_loop = 0
     for (loop, start, end, iters) in build.steps():
+        if loop != in_loop:
+            phases.mark(f"build loop {in_loop} (with its self-recall search)")
+            in_loop = loop
         done += 1
         if done == k_steps:
             t_first_k = time.time() - t_start   # closest_vectors returns after a stream synchronisation
         if time.time() - t_said > 30.0:   # a long build keeps talking
             t_said = time.time()
             log(f"[bench] build: step {done} of {total_steps}, loop {loop}, {t_said - t_start:.0f} s")
+    phases.mark(f"build loop {in_loop} (with its self-recall search)")
     (beams, dists) = build.result()
     torch.cuda.synchronize()
     t_build = time.time() - t_start
@@ -286,6 +308,7 @@ def main():
                 break
         torch.cuda.synchronize()
         r = step_roofline(profile_read(nv, reset=True, enable=0), dim, batch_rows)
+        phases.mark(f"roofline pass, state of loop {li}")
         r.update(loop=li, replayed_batches=replay, build_launches_of_this_loop=int(build.stats[li]["iterations"]),
                  build_seconds_of_this_loop=build.stats[li]["seconds"])
         per_loop.append(r)
@@ -398,6 +421,7 @@ def main():
         (ann.entry_points, ann.configuration["speculative_readahead"]), ann._entry = keep, None
         ok = [r for r in tuned if r["recall_at_10"] >= 0.95]
         result["search_tuned"] = dict(tried=tuned, best=max(ok, key=lambda r: r["qps"]) if ok else None)
+        phases.mark("search leg")
         log(f"[bench] search (dense seeds): {result['search']}")
         log(f"[bench] search (per-query stop): {result['search_per_query_stop']}")
         log(f"[bench] search (tuned): {result['search_tuned']['best']}")
@@ -420,6 +444,8 @@ def main():
         except Exception as e:  # the CPU leg must never take the GPU numbers down with it
             result["cpu_baseline"] = dict(value=None, unit="vectors/s", cores=0, kind="port", sample=f"failed: {e!r}")
 
+    phases.mark("CPU leg (the GPU's side of its comparisons)")
+    result["beam_step_launches_by_phase"] = phases.rows
     print(json.dumps(result), flush=True)
 
 

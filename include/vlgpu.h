@@ -179,7 +179,12 @@ typedef struct vl_beam_params {
     int64_t metric;               /* VL_METRIC_COSINE (the reference's) or VL_METRIC_L2 */
 } vl_beam_params;
 
-/* Forms of one iteration, all with the same result on [:, :queue_length]:
+/* Forms of one iteration, all with the same result on [:, :queue_length] for a
+ * search queue in the state vl_queue_insert leaves it - rows ordered by
+ * (distance, id) with distinct ids - whose distances are the distances of its
+ * ids to this call's query rows (an id carries one distance wherever it
+ * occurs).  Only SORT_MERGE treats a queue in any other state as the
+ * reference does; the other forms are not checked against such input.
  * default        one fused launch (expand + merge phases of a row in one workgroup);
  * TWO_LAUNCHES   expand kernel, then merge kernel;
  * SORT_MERGE     two launches, the merge step sorts whole queue rows (exact for

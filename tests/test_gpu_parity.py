@@ -856,3 +856,36 @@ def test_l2_build_and_search_against_oracle():
     assert rec > 0.8
     with pytest.raises(ValueError):
         ann.search(dev(qv), seeding="dense")
+
+
+def test_self_recall_with_a_sample_that_is_not_the_head_of_the_vectors():
+    """ann_calculate_recall seeds row i with ids over the SAMPLE and distances between sample rows
+    (ann.py:196-208), then searches `vectors`: for a sample taken from the middle an id carries two
+    distances.  The Python layer then picks the whole-row-sort form of the loop; same answer as the oracle."""
+    say("self-recall over a middle slice")
+    from vectorlink_gpu.ann import ann_calculate_recall
+
+    rng = np.random.default_rng(57)
+    n, dim = 1200, 24
+    v = unit(rng, n, dim)
+    c = cfg(beam_size=8, beam_queue_factor=2, recall_search_queue_factor=2)
+    table = orc.generate_circulant_beams(n, orc.primes(8))
+    for (lo, hi) in ((0, 300), (500, 800)):
+        want = orc.ann_calculate_recall(v, table, c, sample=v[lo:hi])
+        got = ann_calculate_recall(dev(v), dev(table), c, sample=dev(v)[lo:hi])
+        assert tuple(got) == tuple(want), (lo, hi)
+
+
+def test_dedup_sort():
+    """utils.dedup_sort (utils.py:85-89): sort, punch out neighbouring duplicates, sort: each row ends up as its
+    distinct ids in ascending order followed by empty ids."""
+    say("dedup_sort")
+    from vectorlink_gpu.utils import dedup_sort
+
+    rng = np.random.default_rng(58)
+    rows = rng.integers(0, 40, (50, 33)).astype(np.int32)
+    rows[3, :5] = M
+    got = host(dedup_sort(dev(rows)))
+    for r in range(rows.shape[0]):
+        distinct = sorted(set(int(x) for x in rows[r] if x != M))
+        assert got[r].tolist() == distinct + [M] * (rows.shape[1] - len(distinct))

@@ -631,9 +631,20 @@ struct StepArgs {
     int dim, nchunks, width;
     uint64_t *memo;
     int memo_shift;
+    int32_t *memo_rate;   // per row: share (x 256) of the candidates of iteration kMemoDecide that were cached
+    int memo_min_rate;    // the cache stays in use only if that share is at least this (x 256)
     int count_evals;
     int l2;  // 0: cosine distance, 1: squared L2
 };
+
+// A probe of the distance cache is a random 8-byte read and every evaluated distance a random 8-byte
+// write - a memory sector each, and one more round trip before the candidate rows can be asked for - so
+// the cache only pays when enough probes hit; how many depends on the row size (short rows are cheap to
+// fetch again).  Each row therefore decides for itself: it uses the cache during its first kMemoDecide - 1
+// iterations, measures the share of hits in iteration kMemoDecide, and leaves the cache alone for the rest
+// of the call if that share is below the break-even share.  A hit returns the bits that would be computed
+// again, so the decision never changes a result.
+constexpr int kMemoDecide = 9;
 
 template <int CPL, int LPR, int U, bool GENERIC, int THREADS>
 __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
@@ -659,7 +670,16 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
     const int32_t *visit = a.v_ids + row * a.VL;
     const float *q_row = s.queries + row * s.dim;
     uint64_t *memo_row = s.memo ? s.memo + ((uint64_t)row << (32 - s.memo_shift)) : nullptr;
-    int n_wanted = 0, n_fetched = 0;  // profiling counts of this wavefront
+    __shared__ int probe_hits_s, probe_asked_s;
+    const bool resample = memo_row && t == kMemoDecide;
+    if (memo_row && t > kMemoDecide && s.memo_rate[row] < s.memo_min_rate) memo_row = nullptr;
+    const bool probing = memo_row != nullptr;
+    if (resample && threadIdx.x == 0) {
+        probe_hits_s = 0;
+        probe_asked_s = 0;
+    }
+    if (resample) __syncthreads();
+    int n_wanted = 0, n_fetched = 0;  // counts of this wavefront
     for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
         const int slot = c0 + lane;
         const bool has = slot < a.m;
@@ -674,15 +694,15 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
             li[slot] = ok ? id : VL_MAXINT;
             if (!ok) ld[slot] = VL_MAXFLOAT;
         }
-        if (s.count_evals) n_wanted += __popcll(__ballot(ok));
-        if (memo_row && ok) {
+        if (s.count_evals || resample) n_wanted += __popcll(__ballot(ok));
+        if (probing && ok) {
             uint64_t e = memo_load(memo_row, s.memo_shift, id);
             if ((int32_t)(uint32_t)e == id) {
                 ld[slot] = __builtin_bit_cast(float, (uint32_t)(e >> 32));
                 ok = false;
             }
         }
-        if (s.count_evals) n_fetched += __popcll(__ballot(ok));
+        if (s.count_evals || resample) n_fetched += __popcll(__ballot(ok));
         if constexpr (GENERIC)
             wave_distances_generic(q_row, s.vectors, s.dim, s.nchunks, id, ok, ld + c0, memo_row, s.memo_shift, s.l2 != 0);
         else
@@ -693,7 +713,13 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
         if (n_wanted) atomicAdd(&c->wanted[stripe], (unsigned long long)n_wanted);
         if (n_fetched) atomicAdd(&c->evals[stripe], (unsigned long long)n_fetched);
     }
+    if (resample && lane == 0) {
+        atomicAdd(&probe_asked_s, n_wanted);
+        atomicAdd(&probe_hits_s, n_wanted - n_fetched);
+    }
     __syncthreads();
+    if (resample && threadIdx.x == 0)
+        s.memo_rate[row] = probe_asked_s > 0 ? (probe_hits_s * 256) / probe_asked_s : 256;
     // ---- merge: ann.py:75-88 ----
     merge_row<THREADS, true>(a, smem);
 }
@@ -707,12 +733,25 @@ void launch_step(const StepArgs &s, int threads, size_t smem, hipStream_t st) {
         hipLaunchKernelGGL((beam_step_kernel<CPL, LPR, U, GENERIC, 256>), grid, dim3(256), smem, st, s);
 }
 
+// VL_DIST_VARIANT (experiments only): 1 = two rows per load for rows of up to 512 bytes (32 lanes each) and
+// one row per load for rows of up to 1536 bytes, the shapes used before lane groups of 16 / 32 took them over.
+int dist_variant() {
+    static const int v = [] {
+        const char *e = getenv("VL_DIST_VARIANT");
+        return e ? atoi(e) : 0;
+    }();
+    return v;
+}
+
 int launch_step_by_dim(const StepArgs &s, bool aligned, int threads, size_t smem, hipStream_t st) {
     const int nchunks = s.nchunks;
+    const int variant = dist_variant();
     if (!aligned || nchunks > 512) launch_step<1, 64, 1, true>(s, threads, smem, st);
     else if (nchunks <= 16) launch_step<1, 16, 8, false>(s, threads, smem, st);
-    else if (nchunks <= 32) launch_step<1, 32, 8, false>(s, threads, smem, st);
+    else if (nchunks <= 32 && variant == 1) launch_step<1, 32, 8, false>(s, threads, smem, st);
+    else if (nchunks <= 32) launch_step<2, 16, 4, false>(s, threads, smem, st);
     else if (nchunks <= 64) launch_step<1, 64, 8, false>(s, threads, smem, st);
+    else if (nchunks <= 96 && variant != 1) launch_step<3, 32, 4, false>(s, threads, smem, st);
     else if (nchunks <= 128) launch_step<2, 64, 8, false>(s, threads, smem, st);
     else if (nchunks <= 192) launch_step<3, 64, 4, false>(s, threads, smem, st);
     else if (nchunks <= 256) launch_step<4, 64, 4, false>(s, threads, smem, st);
@@ -726,7 +765,7 @@ int launch_step_by_dim(const StepArgs &s, bool aligned, int threads, size_t smem
 
 struct BeamLayout {
     int64_t m, VL, Vt, E, head;
-    int64_t off_cand_ids, off_cand_d, off_v_ids, off_v_d, off_seen, off_seen_count, off_row_quiet, off_ctrl, off_memo, total;
+    int64_t off_cand_ids, off_cand_d, off_v_ids, off_v_d, off_seen, off_seen_count, off_row_quiet, off_memo_rate, off_ctrl, off_memo, total;
     int memo_slots;
 };
 
@@ -765,6 +804,7 @@ int beam_layout(const vl_beam_params *p, BeamLayout *l, bool lean = false) {
     l->off_seen = o; o = align256(o + p->n_rows * l->E * 4);
     l->off_seen_count = o; o = align256(o + p->n_rows * 4);
     l->off_row_quiet = o; o = align256(o + p->n_rows * 4);
+    l->off_memo_rate = o; o = align256(o + p->n_rows * 4);
     l->off_ctrl = o; o = align256(o + (int64_t)sizeof(BeamCtrl));
     // per-row cache of evaluated (id, distance) pairs: 128 slots per candidate of one iteration,
     // 1Ki..64Ki per row, the whole table at most 8 GiB (measured at 1M x 768: 16Ki -> 64Ki slots cuts the
@@ -902,6 +942,16 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     step.dim = (int)p->dim; step.nchunks = (int)((p->dim + 3) / 4); step.width = (int)p->width;
     step.l2 = p->metric == VL_METRIC_L2;
     step.memo = l.memo_slots > 0 ? memo : nullptr;
+    step.memo_rate = (int32_t *)(ws + l.off_memo_rate);  // written in iteration kMemoDecide, read after it
+    {
+        // break-even share of hits, measured on 512-byte rows at about 0.4 and scaled with the row size
+        static const int rate_env = [] {
+            const char *e = getenv("VL_BEAM_MEMO_MIN_RATE");
+            return e ? atoi(e) : -1;
+        }();
+        int64_t r = (205ll * 256) / (4 * p->dim);
+        step.memo_min_rate = rate_env >= 0 ? rate_env : (int)(r > 255 ? 255 : r);
+    }
     step.memo_shift = 32;
     if (step.memo) {
         int lg = 0;

@@ -12,10 +12,11 @@
 // CPU oracle produce the same bits): the row is cut into chunks of 4 floats,
 // chunk c belongs to partial sum c mod 64, a partial sum takes its elements in
 // index order with one fused multiply-add each, and the 64 partial sums are
-// folded pairwise at lane distances 32, 16, 8, 4, 2, 1.  Rows of at most
-// 4*LPR floats (LPR = 16 or 32) are handled by groups of LPR lanes, several
-// rows per wavefront; the missing upper partial sums are zeros, so the result
-// is the same.
+// folded pairwise at lane distances 32, 16, 8, 4, 2, 1.  Short rows are
+// handled by groups of LPR = 16 or 32 lanes, several rows per wavefront: a lane
+// then holds the partial sums lig, lig + LPR, ... of its row and folds them
+// itself (distances 32 and 16) before the cross-lane folds; partial sums no
+// chunk reaches are zeros, so the result is the same.
 #include "vl_common.h"
 #include "beam_ctrl.h"
 #include "dist_device.h"
@@ -139,8 +140,9 @@ void launch_expand_piece(const ExpandArgs &a, bool aligned, hipStream_t st) {
     if (!aligned || nchunks > 512) {
         hipLaunchKernelGGL((expand_kernel<1, 64, 1, true>), grid, dim3(256), 0, st, a);
     } else if (nchunks <= 16) launch_fast<1, 16, 8>(a, grid, st);
-    else if (nchunks <= 32) launch_fast<1, 32, 8>(a, grid, st);
+    else if (nchunks <= 32) launch_fast<2, 16, 4>(a, grid, st);
     else if (nchunks <= 64) launch_fast<1, 64, 8>(a, grid, st);
+    else if (nchunks <= 96) launch_fast<3, 32, 4>(a, grid, st);
     else if (nchunks <= 128) launch_fast<2, 64, 8>(a, grid, st);
     else if (nchunks <= 192) launch_fast<3, 64, 4>(a, grid, st);
     else if (nchunks <= 256) launch_fast<4, 64, 4>(a, grid, st);

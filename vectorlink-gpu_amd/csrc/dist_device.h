@@ -123,26 +123,43 @@ __device__ __forceinline__ void wave_distances(const float *__restrict__ q_row,
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            float acc = 0.0f;
+            // Chunk c of a row belongs to partial sum c mod 64.  A lane of an LPR-lane group holds the
+            // chunks lig + LPR * i, i.e. the partial sums lig, lig + LPR, ... (V = 64 / LPR of them, the
+            // (V + j)-th chunk continuing the j-th sum), and folds them at lane distances 32 and 16 itself
+            // before the group's cross-lane folds: the same additions in the same order as 64 lanes with one
+            // partial sum each (sums no chunk reaches are +0).
+            constexpr int V = kWave / LPR;
+            float part[V];
+#pragma unroll
+            for (int j = 0; j < V; ++j) part[j] = 0.0f;
             if (l2) {  // uniform over the launch
 #pragma unroll
                 for (int i = 0; i < CPL; ++i) {
                     const float dx = r[u][i].x - q[i].x, dy = r[u][i].y - q[i].y;
                     const float dz = r[u][i].z - q[i].z, dw = r[u][i].w - q[i].w;
-                    acc = __builtin_fmaf(dx, dx, acc);
-                    acc = __builtin_fmaf(dy, dy, acc);
-                    acc = __builtin_fmaf(dz, dz, acc);
-                    acc = __builtin_fmaf(dw, dw, acc);
+                    float a = part[i % V];
+                    a = __builtin_fmaf(dx, dx, a);
+                    a = __builtin_fmaf(dy, dy, a);
+                    a = __builtin_fmaf(dz, dz, a);
+                    a = __builtin_fmaf(dw, dw, a);
+                    part[i % V] = a;
                 }
             } else {
 #pragma unroll
                 for (int i = 0; i < CPL; ++i) {
-                    acc = __builtin_fmaf(r[u][i].x, q[i].x, acc);
-                    acc = __builtin_fmaf(r[u][i].y, q[i].y, acc);
-                    acc = __builtin_fmaf(r[u][i].z, q[i].z, acc);
-                    acc = __builtin_fmaf(r[u][i].w, q[i].w, acc);
+                    float a = part[i % V];
+                    a = __builtin_fmaf(r[u][i].x, q[i].x, a);
+                    a = __builtin_fmaf(r[u][i].y, q[i].y, a);
+                    a = __builtin_fmaf(r[u][i].z, q[i].z, a);
+                    a = __builtin_fmaf(r[u][i].w, q[i].w, a);
+                    part[i % V] = a;
                 }
             }
+#pragma unroll
+            for (int h = V / 2; h >= 1; h >>= 1)
+#pragma unroll
+                for (int j = 0; j < h; ++j) part[j] = part[j] + part[j + h];
+            float acc = part[0];
             acc = fold_group<LPR>(acc);
             if (lig == 0 && mysrc[u] >= 0) {
                 float d = finish_distance(acc, l2);

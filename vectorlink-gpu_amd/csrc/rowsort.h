@@ -10,11 +10,16 @@ constexpr int kQueueWaves = kQueueThreads / kWave;
 constexpr int kMaxRowSlots = 4096;   // largest row (after padding to a power of two) sorted in LDS
 
 // Ascending bitonic sort of P (power of two) keys in LDS by the whole
-// workgroup.  Ends with a barrier.
+// workgroup.  Ends with a barrier.  A compare-exchange step whose partners lie
+// 64 or more keys apart goes through LDS with a barrier; the steps below that
+// distance stay inside one wavefront's 64 consecutive keys and run in
+// registers (cross-lane exchanges, no barrier), all of them between one LDS
+// read and one LDS write of the key.
 __device__ inline void block_bitonic_sort(uint64_t *keys, int P) {
     __syncthreads();
     for (int k = 2; k <= P; k <<= 1) {
-        for (int j = k >> 1; j > 0; j >>= 1) {
+        int j = k >> 1;
+        for (; j >= kWave; j >>= 1) {
             for (int t = threadIdx.x; t < (P >> 1); t += blockDim.x) {
                 int i = ((t & ~(j - 1)) << 1) | (t & (j - 1));
                 int p = i | j;
@@ -27,6 +32,17 @@ __device__ inline void block_bitonic_sort(uint64_t *keys, int P) {
             }
             __syncthreads();
         }
+        for (int idx = threadIdx.x; idx < P; idx += blockDim.x) {
+            uint64_t key = keys[idx];
+            const bool up = (idx & k) == 0;
+            for (int jj = j; jj > 0; jj >>= 1) {
+                const uint64_t other = __shfl_xor((unsigned long long)key, jj);
+                const bool take_min = ((idx & jj) == 0) == up;
+                key = (take_min == (other < key)) ? other : key;
+            }
+            keys[idx] = key;
+        }
+        __syncthreads();
     }
 }
 

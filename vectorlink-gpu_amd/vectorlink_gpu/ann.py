@@ -16,6 +16,7 @@ from torch import Tensor
 from . import _native as nv
 from .constants import DEVICE, MAXFLOAT, MAXINT
 from .kernels import calculate_distances, gather_distances, knn_exact, optimize_graph, prune_, search_from_seeds
+from . import log as _log
 from .log import log_time
 from .queue import Queue
 from .utils import add_new_to_seen_, generate_circulant_beams, generate_queue_circulants, primes
@@ -139,6 +140,7 @@ def closest_vectors(query_vecs: Tensor, search_queue: Queue, vectors: Tensor, be
         iterations = nv.check(nv.lib().vl_closest_vectors(
             ctypes.byref(p), nv.ptr(query_vecs), nv.ptr(vectors), nv.ptr(beams), nv.ptr(search_queue.indices),
             nv.ptr(search_queue.distances), nv.ptr(excl), nv.ptr(ws), ws.numel(), nv.stream()))
+    _log.BEAM_ITERATIONS += iterations
     return iterations
 
 
@@ -325,6 +327,15 @@ def dense_search_queue(vectors: Tensor, query_vectors: Tensor, config: Dict, ent
     return queue
 
 
+def _flags_for_sample(sample: Tensor, vectors: Tensor) -> int:
+    """initial_queue (ann.py:196-208) seeds row i with ids over the SAMPLE and their distances to
+    sample rows.  When the sample is the head of `vectors` those are also the distances to
+    vectors[id], which is what the loop evaluates, and the default form of the loop applies.  For
+    any other sample an id can carry two different distances, which only the form that sorts whole
+    rows like the reference treats as the reference does."""
+    return 0 if sample.data_ptr() == vectors.data_ptr() else BEAM_SORT_MERGE
+
+
 def ann_calculate_recall(vectors: Tensor, beams: Tensor, config: Dict, sample: Optional[Tensor] = None,
                          verbose: bool = False):
     """reference ann.py:235-259: share of sample rows whose best hit is themselves"""
@@ -332,7 +343,7 @@ def ann_calculate_recall(vectors: Tensor, beams: Tensor, config: Dict, sample: O
         sample = vectors
     (sample_size, _) = sample.size()
     queue = initial_queue(sample.contiguous(), config)
-    closest_vectors(sample, queue, vectors, beams.contiguous(), config)
+    closest_vectors(sample, queue, vectors, beams.contiguous(), config, flags=_flags_for_sample(sample, vectors))
     expected = torch.arange(sample_size, device=vectors.device)
     actual = queue.indices.t()[0]
     found = (expected == actual).sum().item()
@@ -342,12 +353,12 @@ def ann_calculate_recall(vectors: Tensor, beams: Tensor, config: Dict, sample: O
     return (found, found / sample_size)
 
 
-def search_layers(layers, query_vecs: Tensor, search_queue: Queue, vectors: Tensor, config: Dict):
+def search_layers(layers, query_vecs: Tensor, search_queue: Queue, vectors: Tensor, config: Dict, flags: int = 0):
     """reference ann.py:96-106: one beam search per neighbour table, coarse to fine, each starting
     from the queue the previous one left.  Every table is [N, width] over the ids of `vectors`;
     no ids are excluded, because the queries are vectors, not rows of the index."""
     for layer in layers:
-        closest_vectors(query_vecs, search_queue, vectors, layer.contiguous(), config, None)
+        closest_vectors(query_vecs, search_queue, vectors, layer.contiguous(), config, None, flags=flags)
 
 
 def hnsw_calculate_recall(vectors: Tensor, hnsw, config: Dict, sample: Optional[Tensor] = None, verbose: bool = True):
@@ -357,7 +368,7 @@ def hnsw_calculate_recall(vectors: Tensor, hnsw, config: Dict, sample: Optional[
         sample = vectors
     (sample_size, _) = sample.size()
     queue = initial_queue(sample.contiguous(), config)
-    search_layers(hnsw, sample, queue, vectors, config)
+    search_layers(hnsw, sample, queue, vectors, config, flags=_flags_for_sample(sample, vectors))
     expected = torch.arange(sample_size, device=vectors.device)
     found = (expected == queue.indices.t()[0]).sum().item()
     if verbose:
@@ -576,8 +587,6 @@ class ANN:
 
     def dump_logs(self) -> Dict:
         """reference ann.py:479-489 without the nvidia-smi / git shell-outs"""
-        from . import log as _log
-
         out = self.log.copy()
         out["closest_vectors_batch_time"] = _log.CLOSEST_VECTORS_BATCH_TIME
         out["gpu_arch"] = torch.cuda.get_device_name(self.vectors.device)

@@ -11,6 +11,9 @@ from .constants import DEBUG
 
 # longest closest_vectors call seen so far, in wall seconds (read by ANN.dump_logs)
 CLOSEST_VECTORS_BATCH_TIME = 0.0
+# beam-search iterations run by closest_vectors since the import (one kernel launch each in the default form);
+# a profiler's list of launches can be cut into phases with it
+BEAM_ITERATIONS = 0
 
 
 class _Stopwatch:
