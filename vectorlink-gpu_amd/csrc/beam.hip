@@ -356,10 +356,22 @@ __device__ inline uint64_t block_min_key(uint64_t mine, uint64_t *red, int round
     return m;
 }
 
+// Workgroup-wide scalars shared by the expand and merge phases of a row.
+__shared__ int g_n_ex_s;                  // exclusion ids before the row's first empty one
+__shared__ int32_t g_visit_s[kMaxVisit];  // the ids popped from the visit queue in this iteration
+
+// What the fused step has read of a row before its merge phase starts.
+struct RowState {
+    int cnt;    // fill of the row's visited list
+    int first;  // first visited-list column that is free in every row
+};
+
 // FUSED: the candidates of this row are already in LDS (ids at uk, distances behind them,
-// written by the expand phase of the same workgroup) and the loop state has been checked.
+// written by the expand phase of the same workgroup), the loop state has been checked, and
+// the row's queues, visited list, popped ids and exclusions have been placed in LDS by
+// stage_row (the global reads were issued at the start of the kernel).
 template <int THREADS, bool FUSED>
-__device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *smem) {
+__device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *smem, RowState pre = RowState{0, 0}) {
     const int Pc = a.Pc;
     uint64_t *raw = reinterpret_cast<uint64_t *>(smem);  // candidate keys as they arrive
     uint64_t *uk = raw + Pc;                             // the candidates that can matter, then sorted
@@ -372,15 +384,11 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
     uint8_t *fl = reinterpret_cast<uint8_t *>(exl + a.excl_cols);  // per candidate: bit0 wanted, bit1 rest
     __shared__ int wave_cnt[kQueueWaves];
     __shared__ uint64_t red[2 * kQueueWaves];
-    __shared__ int n_ex_s;
     __shared__ int32_t newv[kMaxVisit];
     __shared__ int n_new_s;
     __shared__ int row_changed_s;  // per-query stop: some slot of the search queue's first L changed
+    int &n_ex_s = g_n_ex_s;
 
-    // Every global read of this workgroup is issued up front, before any of them
-    // is waited for: the control words, the candidates, both queues, the popped
-    // ids and the visited list (its fill is at most Vt ids per earlier iteration,
-    // so the row can be fetched without first waiting for the exact count).
     BeamCtrl *c = a.ctrl;
     const int t = a.iter;
     const int64_t row = blockIdx.x;
@@ -396,37 +404,44 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
 
     const int stop = FUSED ? 0 : c->stop;
     const int first_prev = FUSED ? 0 : c->first[(t - 1) % 3];
-    const int first = c->first[t % 3];
-    int cnt = a.seen_count[row];
-    const int seen_bound = min(a.E, a.Vt * (t - 1));
+    const int first = FUSED ? pre.first : c->first[t % 3];
+    int cnt = FUSED ? pre.cnt : a.seen_count[row];
+    // the ids popped at the start of this iteration (queue.py:87-95), before the row is rewritten
+    int32_t popped = VL_MAXINT;
     if constexpr (FUSED) {
         const int32_t *li = reinterpret_cast<const int32_t *>(uk);
         const float *ld = reinterpret_cast<const float *>(li + a.m);
         for (int i = threadIdx.x; i < a.m; i += blockDim.x) raw[i] = vl_make_key(li[i], ld[i]);
+        if (threadIdx.x < kWave && (int)threadIdx.x < a.Vt) popped = g_visit_s[threadIdx.x];
+        if (threadIdx.x == 0) {
+            n_new_s = 0;
+            row_changed_s = 0;
+        }
     } else {
+        // the visited list's fill is at most Vt ids per earlier iteration, so the row can be
+        // fetched without first waiting for the exact count
+        const int seen_bound = min(a.E, a.Vt * (t - 1));
         for (int i = threadIdx.x; i < a.m; i += blockDim.x) raw[i] = vl_make_key(ci[i], cd[i]);
-    }
-    for (int i = threadIdx.x; i < a.L; i += blockDim.x) qa[i] = vl_make_key(qi[i], qd[i]);
-    for (int i = threadIdx.x; i < nva; i += blockDim.x) va[i] = vl_make_key(vi[a.Vt + i], vd[a.Vt + i]);
-    {
-        const int32_t *srow = a.seen + row * a.E;
-        for (int i = threadIdx.x; i < seen_bound; i += blockDim.x) seen_a[i] = srow[i];
-    }
-    // the ids popped at the start of this iteration (queue.py:87-95), before the row is rewritten
-    int32_t popped = VL_MAXINT;
-    if (threadIdx.x < kWave && (int)threadIdx.x < a.Vt) popped = vi[threadIdx.x];
-    if (threadIdx.x == 0) {
-        n_ex_s = a.excl ? a.excl_cols : 0;
-        n_new_s = 0;
-        row_changed_s = 0;
-    }
-    __syncthreads();
-    if (a.excl) {
-        const int32_t *ex = a.excl + row * a.excl_cols;
-        for (int i = threadIdx.x; i < a.excl_cols; i += blockDim.x) {
-            int32_t e = ex[i];
-            exl[i] = e;
-            if (e == VL_MAXINT) atomicMin(&n_ex_s, i);
+        for (int i = threadIdx.x; i < a.L; i += blockDim.x) qa[i] = vl_make_key(qi[i], qd[i]);
+        for (int i = threadIdx.x; i < nva; i += blockDim.x) va[i] = vl_make_key(vi[a.Vt + i], vd[a.Vt + i]);
+        {
+            const int32_t *srow = a.seen + row * a.E;
+            for (int i = threadIdx.x; i < seen_bound; i += blockDim.x) seen_a[i] = srow[i];
+        }
+        if (threadIdx.x < kWave && (int)threadIdx.x < a.Vt) popped = vi[threadIdx.x];
+        if (threadIdx.x == 0) {
+            n_ex_s = a.excl ? a.excl_cols : 0;
+            n_new_s = 0;
+            row_changed_s = 0;
+        }
+        __syncthreads();
+        if (a.excl) {
+            const int32_t *ex = a.excl + row * a.excl_cols;
+            for (int i = threadIdx.x; i < a.excl_cols; i += blockDim.x) {
+                int32_t e = ex[i];
+                exl[i] = e;
+                if (e == VL_MAXINT) atomicMin(&n_ex_s, i);
+            }
         }
     }
     if (stop) return;
@@ -483,7 +498,10 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
     // ---- which candidates can matter at all -------------------------------------------
     // search queue: only keys below its last slot can enter.  visit queue (VL slots, Vt of
     // them just freed): every unvisited key below its last live slot, plus the Vt best
-    // distinct unvisited keys above it.  Everything else is dropped before the sort.
+    // distinct unvisited keys above it.  Everything else is dropped before the sort.  What is
+    // chosen here may be a superset - the merges below are exact and cut by rank - so the keys
+    // above the visit queue's last slot ("rest") are looked up in the visited list only when
+    // they come up as one of the smallest.
     const uint64_t ws = qa[a.L - 1];
     const uint64_t wv = nva > 0 ? va[nva - 1] : 0ull;
     for (int i = threadIdx.x; i < a.m; i += blockDim.x) {
@@ -629,6 +647,7 @@ struct StepArgs {
     const int32_t *beams;
     int64_t n_vectors;
     int dim, nchunks, width;
+    uint32_t width_magic;  // floor(2^32 / width) + 1: slot / width == umulhi(slot, width_magic) for slot * width < 2^32
     uint64_t *memo;
     int memo_shift;
     int32_t *memo_rate;   // per row: share (x 256) of the candidates of iteration kMemoDecide that were cached
@@ -646,49 +665,140 @@ struct StepArgs {
 // again, so the decision never changes a result.
 constexpr int kMemoDecide = 9;
 
+// Elements of a row that one thread brings in at the start of the fused step and keeps in registers until
+// the workgroup's other reads have been issued: search queue, visit queue, visited list.  Longer rows load
+// their remainder the slow way (read, wait, store) - none of the benchmark shapes has one.
+constexpr int kPreQ = 2, kPreV = 2, kPreS = 4;
+
 template <int CPL, int LPR, int U, bool GENERIC, int THREADS>
 __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
     extern __shared__ __align__(16) unsigned char smem[];
     const MergeArgs &a = s.m;
     BeamCtrl *c = a.ctrl;
     const int t = a.iter;
-    const int gate = beam_gate(c, t, a.readahead, a.E, blockIdx.x == 0 && threadIdx.x == 0);
-    if (gate == 2) return;
+    const int tid = threadIdx.x;
     const int64_t row = blockIdx.x;
-    if (gate == 1 || (a.row_quiet && a.row_quiet[row] >= a.readahead)) {
+    // ---- every read that depends on nothing else goes out first: loop state, the row's counters, the ids
+    // to visit, both queues, the visited list, the exclusions.  A round trip to memory costs more than
+    // anything this workgroup computes, so the number of dependent round trips is what it pays for: this
+    // one, then the neighbour lists of the visited ids, the cache probes, the candidate rows.
+    int32_t *vi = a.v_ids + row * a.VL;
+    float *vd = a.v_d + row * a.VL;
+    const int32_t *qi = a.q_ids + row * a.cap;
+    const float *qd = a.q_d + row * a.cap;
+    const int32_t *srow = a.seen + row * a.E;
+    const int nva = a.VL - a.Vt;
+    const int seen_bound = min(a.E, a.Vt * (t - 1));  // the fill is at most Vt ids per earlier iteration
+    const int32_t my_visit = tid < a.Vt ? vi[tid] : VL_MAXINT;
+    RowState pre;
+    pre.cnt = a.seen_count[row];
+    pre.first = c->first[t % 3];
+    const int quiet = a.row_quiet ? a.row_quiet[row] : 0;
+    const int memo_rate = (s.memo && t > kMemoDecide) ? s.memo_rate[row] : 256;
+    int32_t pq_i[kPreQ], pv_i[kPreV], ps[kPreS];
+    float pq_d[kPreQ], pv_d[kPreV];
+#pragma unroll
+    for (int j = 0; j < kPreQ; ++j) {
+        const int i = tid + j * THREADS;
+        pq_i[j] = i < a.L ? qi[i] : VL_MAXINT;
+        pq_d[j] = i < a.L ? qd[i] : VL_MAXFLOAT;
+    }
+#pragma unroll
+    for (int j = 0; j < kPreV; ++j) {
+        const int i = tid + j * THREADS;
+        pv_i[j] = i < nva ? vi[a.Vt + i] : VL_MAXINT;
+        pv_d[j] = i < nva ? vd[a.Vt + i] : VL_MAXFLOAT;
+    }
+#pragma unroll
+    for (int j = 0; j < kPreS; ++j) {
+        const int i = tid + j * THREADS;
+        ps[j] = i < seen_bound ? srow[i] : VL_MAXINT;
+    }
+    int32_t my_excl = VL_MAXINT;
+    if (a.excl && tid < a.excl_cols) my_excl = a.excl[row * a.excl_cols + tid];
+
+    const int gate = beam_gate(c, t, a.readahead, a.E, blockIdx.x == 0 && tid == 0);
+    if (gate == 2) return;
+    if (gate == 1 || (a.row_quiet && quiet >= a.readahead)) {
         // the visit queue is no longer fed (every candidate of this iteration is empty), or this row has
         // stopped on its own: nothing changes, only the running maximum is kept current
-        if (threadIdx.x == 0) raise_running_max(&c->first[(t + 1) % 3], a.seen_count[row], min(a.E, a.Vt * t));
+        if (tid == 0) raise_running_max(&c->first[(t + 1) % 3], pre.cnt, min(a.E, a.Vt * t));
         return;
     }
-    // ---- expand: ann.py:69-73 (pop the visit heads, gather their neighbour lists, distances) ----
-    uint64_t *uk = reinterpret_cast<uint64_t *>(smem) + a.Pc;
+    uint64_t *raw = reinterpret_cast<uint64_t *>(smem);
+    uint64_t *uk = raw + a.Pc;
+    uint64_t *qa = uk + 2 * a.Pc;
+    uint64_t *va = qa + a.L;
+    int32_t *seen_a = reinterpret_cast<int32_t *>(va + a.VL);
+    int32_t *exl = seen_a + 2 * a.E;
     int32_t *li = reinterpret_cast<int32_t *>(uk);
     float *ld = reinterpret_cast<float *>(li + a.m);
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
-    const int32_t *visit = a.v_ids + row * a.VL;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
     const float *q_row = s.queries + row * s.dim;
     uint64_t *memo_row = s.memo ? s.memo + ((uint64_t)row << (32 - s.memo_shift)) : nullptr;
     __shared__ int probe_hits_s, probe_asked_s;
     const bool resample = memo_row && t == kMemoDecide;
-    if (memo_row && t > kMemoDecide && s.memo_rate[row] < s.memo_min_rate) memo_row = nullptr;
+    if (memo_row && memo_rate < s.memo_min_rate) memo_row = nullptr;
     const bool probing = memo_row != nullptr;
-    if (resample && threadIdx.x == 0) {
+    if (tid < a.Vt) g_visit_s[tid] = my_visit;
+    if (tid == 0) {
+        g_n_ex_s = a.excl ? a.excl_cols : 0;
         probe_hits_s = 0;
         probe_asked_s = 0;
     }
-    if (resample) __syncthreads();
-    int n_wanted = 0, n_fetched = 0;  // counts of this wavefront
-    for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
+    __syncthreads();
+
+    // ---- expand: ann.py:69-73 (pop the visit heads, gather their neighbour lists, distances) ----
+    // candidate id of slot c0 + lane: the neighbour list of a visited node
+    auto resolve = [&](int c0) -> int32_t {
         const int slot = c0 + lane;
-        const bool has = slot < a.m;
         int32_t id = VL_MAXINT;
-        if (has) {
-            int sidx = slot / s.width, k = slot - sidx * s.width;
-            int32_t node = visit[sidx];
+        if (slot < a.m) {
+            int sidx = s.width == 1 ? slot : (int)__umulhi((uint32_t)slot, s.width_magic), k = slot - sidx * s.width;
+            int32_t node = g_visit_s[sidx];
             if (node != VL_MAXINT && (uint32_t)node < (uint64_t)s.n_vectors) id = s.beams[(int64_t)node * s.width + k];
         }
+        return id;
+    };
+    int32_t id = resolve(wave * kWave);
+    // The row's own state, read at the top, goes to LDS now that the first neighbour lists are on their
+    // way.  (Outside the loop below on purpose: inside it, its addresses would be kept in registers across
+    // the distance code.)
+    {
+#pragma unroll
+        for (int j = 0; j < kPreQ; ++j) {
+            const int i = tid + j * THREADS;
+            if (i < a.L) qa[i] = vl_make_key(pq_i[j], pq_d[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < kPreV; ++j) {
+            const int i = tid + j * THREADS;
+            if (i < nva) va[i] = vl_make_key(pv_i[j], pv_d[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < kPreS; ++j) {
+            const int i = tid + j * THREADS;
+            if (i < seen_bound) seen_a[i] = ps[j];
+        }
+        if (a.excl && tid < a.excl_cols) {
+            exl[tid] = my_excl;
+            if (my_excl == VL_MAXINT) atomicMin(&g_n_ex_s, tid);
+        }
+        for (int i = tid + kPreQ * THREADS; i < a.L; i += THREADS) qa[i] = vl_make_key(qi[i], qd[i]);
+        for (int i = tid + kPreV * THREADS; i < nva; i += THREADS) va[i] = vl_make_key(vi[a.Vt + i], vd[a.Vt + i]);
+        for (int i = tid + kPreS * THREADS; i < seen_bound; i += THREADS) seen_a[i] = srow[i];
+        for (int i = tid + THREADS; i < a.excl_cols; i += THREADS) {
+            int32_t e = a.excl[row * a.excl_cols + i];
+            exl[i] = e;
+            if (e == VL_MAXINT) atomicMin(&g_n_ex_s, i);
+        }
+    }
+    int n_wanted = 0, n_fetched = 0;  // counts of this wavefront
+    for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
+        if (c0 != wave * kWave) id = resolve(c0);
+        const int slot = c0 + lane;
+        const bool has = slot < a.m;
         bool ok = has && id != VL_MAXINT && id >= 0 && (int64_t)id < s.n_vectors;
         if (has) {
             li[slot] = ok ? id : VL_MAXINT;
@@ -718,10 +828,10 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
         atomicAdd(&probe_hits_s, n_wanted - n_fetched);
     }
     __syncthreads();
-    if (resample && threadIdx.x == 0)
+    if (resample && tid == 0)
         s.memo_rate[row] = probe_asked_s > 0 ? (probe_hits_s * 256) / probe_asked_s : 256;
     // ---- merge: ann.py:75-88 ----
-    merge_row<THREADS, true>(a, smem);
+    merge_row<THREADS, true>(a, smem, pre);
 }
 
 template <int CPL, int LPR, int U, bool GENERIC>
@@ -940,6 +1050,7 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     StepArgs step;
     step.queries = queries; step.vectors = vectors; step.beams = beams; step.n_vectors = p->n_vectors;
     step.dim = (int)p->dim; step.nchunks = (int)((p->dim + 3) / 4); step.width = (int)p->width;
+    step.width_magic = (uint32_t)((1ull << 32) / (uint64_t)p->width + 1);  // not used for width 1 (it does not fit)
     step.l2 = p->metric == VL_METRIC_L2;
     step.memo = l.memo_slots > 0 ? memo : nullptr;
     step.memo_rate = (int32_t *)(ws + l.off_memo_rate);  // written in iteration kMemoDecide, read after it
