@@ -221,6 +221,8 @@ def main():
     ap.add_argument("--no-search", action="store_true", help="skip the search leg")
     ap.add_argument("--cpu-rows", type=int, default=768)
     ap.add_argument("--loops", type=int, default=3, help="optimisation loops of the build (the reference's default is 3)")
+    ap.add_argument("--concurrent-batches", type=int, default=4,
+                    help="batches of an optimisation loop kept in flight by the timed build (streams / host threads)")
     ap.add_argument("--prune", choices=["reference", "rank", "none"], default="reference",
                     help="reference = prune_ between loops as the reference does (default); rank = detour-count "
                          "cut with reverse edges at the end (an addition); none = no pruning")
@@ -270,7 +272,7 @@ def main():
     profile_read(nv, reset=True, enable=0)
     torch.cuda.synchronize()
     t_start = time.time()
-    build = GraphBuild(vectors, cfg, keep_history=True)
+    build = GraphBuild(vectors, cfg, keep_history=True, concurrent_batches=args.concurrent_batches)
     total_steps = build.batches_per_loop() * cfg["optimization_loops"]
     k_steps = args.steps if 0 < args.steps < total_steps else total_steps
     done = 0
@@ -302,7 +304,7 @@ def main():
     per_loop = []
     for li, tables in enumerate(build.history):
         profile_read(nv, reset=True, enable=1)
-        rb = GraphBuild(vectors, cfg, initial=tables)
+        rb = GraphBuild(vectors, cfg, initial=tables, concurrent_batches=1)  # one launch at a time under the events
         for i, _ in enumerate(rb.steps()):
             if i + 1 >= replay:
                 break
@@ -342,6 +344,7 @@ def main():
                    "build_queue": cfg["beam_size"] * cfg["beam_queue_factor"], "batch_size": cfg["batch_size"],
                    "optimization_loops": cfg["optimization_loops"], "parallel_visit_count": 4,
                    "prune": args.prune, "build_seeding": "circulant (reference)",
+                   "concurrent_batches": args.concurrent_batches,
                    "search_seeding": "dense, 32768 entry points", "queries": int(queries.shape[0])},
         "partial": False, "build_seconds": t_build, "build_steps": done,
         "steps_note": f"value = n / build_seconds over all {done} steps (hooks off); steps and ms_per_step describe "
@@ -407,20 +410,24 @@ def main():
             seeding_tiles=dict(bound="mfma", seconds=t_seed, tflops=seed_flops / t_seed / 1e12,
                                frac=seed_flops / t_seed / 1e12 / MFMA_FP32_PEAK,
                                entry_points=int(entry_vectors.shape[0])))
-        # the same graph searched with cheaper settings (fewer entry points, shorter queue, a progress check
-        # every second iteration): the fastest of them that still reaches recall@10 >= 0.95
+        # the same graph searched with other settings of the additions (entry points of the dense seeding, queue
+        # length, how often progress is checked, which stop): the fastest of them that still reaches recall@10 >= 0.95
         tuned = []
         keep = (ann.entry_points, ann.configuration["speculative_readahead"])
-        for entry_points in (16_384, 8_192):
-            for qs in (10, 16):
-                ann.entry_points, ann._entry = entry_points, None
-                ann.configuration["speculative_readahead"] = 2
-                r = one_search(qs, "dense", "batch")
-                r.update(entry_points=entry_points, speculative_readahead=2)
-                tuned.append(r)
+        for entry_points in (32_768, 16_384, 8_192, 4_096):
+            for readahead in (2, 5):
+                for qs in (10, 16, 32):
+                    for mode in ("batch", "per_query"):
+                        ann.entry_points, ann._entry = entry_points, None
+                        ann.configuration["speculative_readahead"] = readahead
+                        r = one_search(qs, "dense", mode)
+                        r.update(entry_points=entry_points, speculative_readahead=readahead, stop=mode)
+                        tuned.append(r)
         (ann.entry_points, ann.configuration["speculative_readahead"]), ann._entry = keep, None
         ok = [r for r in tuned if r["recall_at_10"] >= 0.95]
-        result["search_tuned"] = dict(tried=tuned, best=max(ok, key=lambda r: r["qps"]) if ok else None)
+        result["search_tuned"] = dict(tried=tuned, best=max(ok, key=lambda r: r["qps"]) if ok else None,
+                                      best_with_the_reference_stop=max(
+                                          (r for r in ok if r["stop"] == "batch"), key=lambda r: r["qps"], default=None))
         phases.mark("search leg")
         log(f"[bench] search (dense seeds): {result['search']}")
         log(f"[bench] search (per-query stop): {result['search_per_query_stop']}")

@@ -889,3 +889,20 @@ def test_dedup_sort():
     for r in range(rows.shape[0]):
         distinct = sorted(set(int(x) for x in rows[r] if x != M))
         assert got[r].tolist() == distinct + [M] * (rows.shape[1] - len(distinct))
+
+
+def test_build_does_not_depend_on_the_batches_in_flight():
+    """GraphBuild keeps several batches of a loop in flight on streams of their own; one, two and three give
+    the same graph, the oracle's."""
+    say("build with 1, 2, 3 batches in flight")
+    from vectorlink_gpu.ann import generate_ann
+
+    rng = np.random.default_rng(61)
+    n, dim = 4000, 20
+    v = unit(rng, n, dim)
+    c = cfg(beam_size=8, beam_queue_factor=2, batch_size=700, optimization_loops=2)
+    (wb, wd) = orc.generate_ann(v, c)
+    for lanes in (1, 2, 3):
+        (gb, gd) = generate_ann(dev(v), c, concurrent_batches=lanes)
+        assert np.array_equal(host(gb), wb), lanes
+        assert np.array_equal(bits(host(gd)), bits(wd)), lanes

@@ -140,7 +140,8 @@ def closest_vectors(query_vecs: Tensor, search_queue: Queue, vectors: Tensor, be
         iterations = nv.check(nv.lib().vl_closest_vectors(
             ctypes.byref(p), nv.ptr(query_vecs), nv.ptr(vectors), nv.ptr(beams), nv.ptr(search_queue.indices),
             nv.ptr(search_queue.distances), nv.ptr(excl), nv.ptr(ws), ws.numel(), nv.stream()))
-    _log.BEAM_ITERATIONS += iterations
+    with _WORKSPACES_LOCK:
+        _log.BEAM_ITERATIONS += iterations
     return iterations
 
 
@@ -163,13 +164,16 @@ class GraphBuild:
     fused loop relies on an id always carrying the same distance)."""
 
     def __init__(self, vectors: Tensor, config: Dict, stale_distances: bool = False,
-                 initial: Optional[Tuple[Tensor, Tensor]] = None, keep_history: bool = False):
+                 initial: Optional[Tuple[Tensor, Tensor]] = None, keep_history: bool = False,
+                 concurrent_batches: int = 4):
         """initial: (ids, distances) tables of the build-queue width to start from instead of the
         circulant graph (a later optimisation loop's starting state).  keep_history: keep a
         reference to the tables every optimisation loop started from in self.history."""
         self.vectors = vectors
         self.config = config
         self.stale = stale_distances
+        self.concurrent = concurrent_batches  # batches of a loop kept in flight (see steps)
+        self._streams = None
         (self.num_vecs, _) = vectors.size()
         device = vectors.device
         self.beam_size = config["beam_size"]
@@ -204,16 +208,34 @@ class GraphBuild:
                 self.history.append((self.beams, self.beam_distances if self.stale else self.distances))
             next_beams = torch.empty_like(self.beams)
             next_beam_distances = torch.empty_like(self.beam_distances)
-            for start in range(0, self.num_vecs, batch_size):
+            seed_distances = self.beam_distances if self.stale else self.distances
+
+            def run_batch(start: int, stream) -> int:
                 end = min(start + batch_size, self.num_vecs)
-                exclude = excluding_self(start, end, ql, device)
-                queue = Queue(end - start, ql, ql + remaining_capacity, device=device)
-                seed_distances = self.beam_distances if self.stale else self.distances
-                queue.insert(self.beams.narrow(0, start, end - start), seed_distances.narrow(0, start, end - start))
-                t = search(vectors[start:end], queue, vectors, self.beams, config, exclude)
+                with torch.cuda.stream(stream):
+                    exclude = excluding_self(start, end, ql, device)
+                    queue = Queue(end - start, ql, ql + remaining_capacity, device=device)
+                    queue.insert(self.beams.narrow(0, start, end - start), seed_distances.narrow(0, start, end - start))
+                    t = search(vectors[start:end], queue, vectors, self.beams, config, exclude)
+                    next_beams.narrow(0, start, end - start).copy_(queue.indices.narrow(1, 0, ql))
+                    next_beam_distances.narrow(0, start, end - start).copy_(queue.distances.narrow(1, 0, ql))
+                    stream.synchronize()
+                return t
+
+            # The batches of a loop only read the previous loop's table and write disjoint rows of the next
+            # one (ann.py:132-166), so `concurrent` of them are kept in flight, each on a stream and a host
+            # thread of its own: while one batch's launch drains, the other's fills the idle compute units.
+            # The result does not depend on it.
+            starts = list(range(0, self.num_vecs, batch_size))
+            lanes = max(1, min(self.concurrent, len(starts)))
+            torch.cuda.synchronize(device)  # the tables come from the main stream
+            if lanes == 1:
+                results = ((start, run_batch(start, torch.cuda.current_stream(device))) for start in starts)
+            else:
+                results = self._in_flight(run_batch, starts, lanes, device)
+            for (start, t) in results:
+                end = min(start + batch_size, self.num_vecs)
                 iterations += t
-                next_beams.narrow(0, start, end - start).copy_(queue.indices.narrow(1, 0, ql))
-                next_beam_distances.narrow(0, start, end - start).copy_(queue.distances.narrow(1, 0, ql))
                 last = end == self.num_vecs
                 if last:
                     recall = self._finish_loop(next_beams, next_beam_distances)
@@ -224,6 +246,24 @@ class GraphBuild:
             if recall == 1.0:  # ann.py:187
                 break
         self.finished = True
+
+    def _in_flight(self, run_batch, starts, lanes: int, device):
+        """Runs run_batch(start, stream) for every start with `lanes` of them in flight, yielding
+        (start, result) in the order of `starts`."""
+        from concurrent.futures import ThreadPoolExecutor
+
+        if self._streams is None or len(self._streams) < lanes:
+            self._streams = [torch.cuda.Stream(device=device) for _ in range(lanes)]
+        with ThreadPoolExecutor(max_workers=lanes) as pool:
+            pending = []
+            for k, start in enumerate(starts):
+                if len(pending) == lanes:
+                    (s0, f0) = pending.pop(0)
+                    yield (s0, f0.result())
+                # batch k runs on stream k % lanes, free again because batch k - lanes has been waited for
+                pending.append((start, pool.submit(run_batch, start, self._streams[k % lanes])))
+            for (s0, f0) in pending:
+                yield (s0, f0.result())
 
     def _finish_loop(self, next_beams: Tensor, next_beam_distances: Tensor) -> float:
         if self.config["prune"] is True:  # ann.py:171-177 (prune="rank" thins nothing between loops)
@@ -245,11 +285,11 @@ class GraphBuild:
 
 
 def generate_ann(vectors: Tensor, config: Dict, stale_distances: bool = False,
-                 stats: Optional[list] = None) -> Tuple[Tensor, Tensor]:
+                 stats: Optional[list] = None, concurrent_batches: int = 4) -> Tuple[Tensor, Tensor]:
     """reference ann.py:109-193 (see GraphBuild).  stats, when given, receives
     one dict per optimisation loop (wall seconds, beam-search iterations summed
     over batches, self-recall)."""
-    build = GraphBuild(vectors, config, stale_distances)
+    build = GraphBuild(vectors, config, stale_distances, concurrent_batches=concurrent_batches)
     for _ in build.steps():
         pass
     if stats is not None:
@@ -412,6 +452,7 @@ class ANN:
         entry_points: int = 32_768,
         keep_queues: bool = False,
         metric: str = "cosine",
+        concurrent_batches: int = 4,
     ):
         """seeding / entry_points are additions: "circulant" seeds searches as the
         reference does; "dense" seeds them from the nearest of `entry_points`
@@ -419,7 +460,9 @@ class ANN:
         "rank": no pruning between loops, and the final cut from the build queue
         width to beam_size is done by detour count with reverse edges merged in
         (kernels.optimize_graph) instead of keeping the first beam_size columns.
-        metric is an addition too: "cosine" is the reference's distance; "l2" builds
+        concurrent_batches (an addition) is the number of batches of an optimisation loop
+        that the build keeps in flight, each on its own stream and host thread; the
+        graph does not depend on it.  metric is an addition too: "cosine" is the reference's distance; "l2" builds
         and searches by squared Euclidean distance (rows need not be unit length;
         the dense seeding and recall_at_k tiles are cosine only and refuse it)."""
         assert prune in (True, False, "rank")
@@ -457,7 +500,7 @@ class ANN:
             else:
                 self.distances = distances.to(self.vectors.device).contiguous()
         else:
-            build = GraphBuild(self.vectors, self.configuration)
+            build = GraphBuild(self.vectors, self.configuration, concurrent_batches=concurrent_batches)
             for _ in build.steps():
                 pass
             self.build_stats: list = build.stats
