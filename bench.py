@@ -41,11 +41,14 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E bandwidth
 MFMA_FP32_PEAK = 157.3  # MI355X published dense fp32 matrix TFLOP/s
 
-# Bytes moved past L2 per launch of the beam-search step, carried over from two rocprofv3 --pmc runs of an
-# earlier build of this workload (FETCH_SIZE x 2.0 after calibration against a 1 GiB copy, + WRITE_SIZE x 1.0);
-# NOT measured in this run.  profiles/beam_step_kernel_mix-1m-768_hbm_traffic.txt holds the runs.
-TRAFFIC = {"mix-1m-768": dict(bytes_per_launch=12.26e9, algorithmic_bytes_per_launch_in_that_run=11.79e9,
-                              scope="first 104 build steps (25,605 launches), from the committed profile, not this run")}
+# Bytes moved past L2 per launch of the beam-search step, per optimisation-loop state, carried over from the
+# rocprofv3 --pmc runs of this same command that profiles/beam_step_kernel_<workload>_by_phase.txt records
+# (FETCH_SIZE x 2.0 after calibration against the 1 GiB copy + WRITE_SIZE x 1.0, "roofline pass" phases);
+# NOT measured in this run.  Workloads without a recorded counter run report null.
+TRAFFIC_PER_LOOP = {
+    "mix-1m-768": [(5690637.7 * 2 + 150253.8) * 1024, (1330719.0 * 2 + 56741.5) * 1024, (407900.7 * 2 + 24904.0) * 1024],
+    "mix-1m-128": [(436666.3 * 2 + 25910.0) * 1024, (231534.4 * 2 + 28947.1) * 1024, (153222.4 * 2 + 20410.1) * 1024],
+}
 
 
 def log(*a):
@@ -320,11 +323,21 @@ def main():
     w_bytes = sum(wt * r["algorithmic_bytes_per_launch"] for wt, r in zip(weights, per_loop))
     w_launch = max(sum(weights), 1)
     achieved = w_bytes / (w_time / 1e3) / 1e9 if w_time > 0 else 0.0
+    per_loop_traffic = TRAFFIC_PER_LOOP.get(args.workload)
+    traffic = traffic_detail = None
+    if per_loop_traffic and len(per_loop_traffic) >= len(per_loop) and args.n is None:
+        traffic = sum(wt * tb for wt, tb in zip(weights, per_loop_traffic)) / w_launch
+        traffic_detail = dict(
+            source=f"profiles/beam_step_kernel_{args.workload}_by_phase.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of "
+                   "this command, committed); not measured in this run",
+            bytes_per_launch_by_loop=per_loop_traffic[:len(per_loop)],
+            over_algorithmic_by_loop=[tb / max(r["algorithmic_bytes_per_launch"], 1.0)
+                                      for tb, r in zip(per_loop_traffic, per_loop)])
     roofline = dict(
         bound="hbm",
         kernel="beam_step_kernel (one beam-search iteration: gathered cosine distances + queue merge per row)",
         achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
-        traffic=(TRAFFIC.get(args.workload) or {}).get("bytes_per_launch"), traffic_detail=TRAFFIC.get(args.workload),
+        traffic=traffic, traffic_detail=traffic_detail,
         copy_gbs_measured=copy_gbs, frac_of_measured_copy=achieved / copy_gbs if copy_gbs > 0 else None,
         avg_launch_ms=w_time / w_launch, algorithmic_bytes_per_launch=w_bytes / w_launch,
         launches_in_timed_build=int(sum(weights)),
@@ -413,17 +426,21 @@ def main():
         # the same graph searched with other settings of the additions (entry points of the dense seeding, queue
         # length, how often progress is checked, which stop): the fastest of them that still reaches recall@10 >= 0.95
         tuned = []
-        keep = (ann.entry_points, ann.configuration["speculative_readahead"])
+        keep = (ann.entry_points, ann.configuration["speculative_readahead"], ann.seed_dims)
         for entry_points in (32_768, 16_384, 8_192, 4_096):
-            for readahead in (2, 5):
-                for qs in (10, 16, 32):
-                    for mode in ("batch", "per_query"):
-                        ann.entry_points, ann._entry = entry_points, None
-                        ann.configuration["speculative_readahead"] = readahead
-                        r = one_search(qs, "dense", mode)
-                        r.update(entry_points=entry_points, speculative_readahead=readahead, stop=mode)
-                        tuned.append(r)
-        (ann.entry_points, ann.configuration["speculative_readahead"]), ann._entry = keep, None
+            for seed_dims in (None, 256 if dim > 256 else None, 128 if dim > 128 else None):
+                if seed_dims is None and (entry_points, None) in {(t["entry_points"], t["seed_dims"]) for t in tuned}:
+                    continue
+                for readahead in (2, 5):
+                    for qs in (10, 16, 32):
+                        for mode in ("batch", "per_query"):
+                            ann.entry_points, ann.seed_dims, ann._entry = entry_points, seed_dims, None
+                            ann.configuration["speculative_readahead"] = readahead
+                            r = one_search(qs, "dense", mode)
+                            r.update(entry_points=entry_points, seed_dims=seed_dims, speculative_readahead=readahead,
+                                     stop=mode)
+                            tuned.append(r)
+        (ann.entry_points, ann.configuration["speculative_readahead"], ann.seed_dims), ann._entry = keep, None
         ok = [r for r in tuned if r["recall_at_10"] >= 0.95]
         result["search_tuned"] = dict(tried=tuned, best=max(ok, key=lambda r: r["qps"]) if ok else None,
                                       best_with_the_reference_stop=max(

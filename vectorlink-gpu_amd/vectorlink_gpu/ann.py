@@ -348,6 +348,9 @@ def entry_point_ids(vector_count: int, entry_points: int, device=DEVICE) -> Tens
 
 def dense_search_queue(vectors: Tensor, query_vectors: Tensor, config: Dict, entry_ids: Tensor,
                        entry_vectors: Tensor, queue_size: Optional[int] = None) -> Queue:
+    # entry_vectors may hold only the first columns of the entry points (ANN.seed_dims): the seeds are
+    # then ranked by that part of the dot product, which is enough to land near the query; the distances
+    # that enter the queue are always the full ones.
     """Query-dependent seeding (not in the reference, whose seeds (b + p_k) % N ignore
     the query, utils.py:26-32): the seeds of a query are its DENSE_SEEDS nearest
     entry points, found with one dense query x entry-point pass on fp32 MFMA tiles.
@@ -360,7 +363,9 @@ def dense_search_queue(vectors: Tensor, query_vectors: Tensor, config: Dict, ent
     extra_capacity = max(queue_size, config["parallel_visit_count"] * config["beam_size"])
     queue = Queue(batch_size, queue_size, queue_size + extra_capacity, device=vectors.device)
     k = min(DENSE_SEEDS, entry_ids.size(0), queue_size)
-    (local, _) = knn_exact(query_vectors, entry_vectors, k)
+    cols = entry_vectors.size(1)
+    ranked_by = query_vectors if cols == query_vectors.size(1) else query_vectors[:, :cols].contiguous()
+    (local, _) = knn_exact(ranked_by, entry_vectors, k)
     seeds = entry_ids[local.long()].contiguous()
     d = query_cosine_distances(query_vectors, vectors, seeds, config.get("metric", "cosine"))
     queue.insert(seeds, d)
@@ -453,6 +458,7 @@ class ANN:
         keep_queues: bool = False,
         metric: str = "cosine",
         concurrent_batches: int = 4,
+        seed_dims: Optional[int] = None,
     ):
         """seeding / entry_points are additions: "circulant" seeds searches as the
         reference does; "dense" seeds them from the nearest of `entry_points`
@@ -460,6 +466,8 @@ class ANN:
         "rank": no pruning between loops, and the final cut from the build queue
         width to beam_size is done by detour count with reverse edges merged in
         (kernels.optimize_graph) instead of keeping the first beam_size columns.
+        seed_dims (with seeding="dense") ranks the entry points by their first seed_dims
+        columns only - a cheaper pass that still lands near the query; None uses all.
         concurrent_batches (an addition) is the number of batches of an optimisation loop
         that the build keeps in flight, each on its own stream and host thread; the
         graph does not depend on it.  metric is an addition too: "cosine" is the reference's distance; "l2" builds
@@ -472,6 +480,8 @@ class ANN:
         assert seeding in ("circulant", "dense")
         self.seeding = seeding
         self.entry_points = entry_points
+        self.seed_dims = seed_dims
+        assert seed_dims is None or (seed_dims > 0 and seed_dims % 4 == 0), "seed_dims must be a multiple of 4"
         self._entry = None
         self._queues = None
         (count, dim) = vectors.size()
@@ -581,7 +591,10 @@ class ANN:
     def _entry_tables(self):
         if self._entry is None:
             ids = entry_point_ids(self.vectors.size(0), self.entry_points, self.vectors.device)
-            self._entry = (ids, self.vectors[ids.long()].contiguous())
+            rows = self.vectors[ids.long()]
+            if self.seed_dims is not None and self.seed_dims < rows.size(1):
+                rows = rows[:, :self.seed_dims]
+            self._entry = (ids, rows.contiguous())
         return self._entry
 
     def search(self, query: Tensor, queue_size: Optional[int] = None, seeding: Optional[str] = None,
