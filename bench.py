@@ -78,6 +78,24 @@ def step_roofline(prof, dim, batch_rows):
                 distances_served_from_cache=1.0 - prof["evals"] / max(prof["wanted"], 1.0))
 
 
+def measured_read_gbs(torch, dev):
+    """Bandwidth of a read-only pass (a sum) over 4 GiB of device memory, best of 5."""
+    src = torch.empty(1 << 30, dtype=torch.float32, device=dev).fill_(1.0)
+    src.sum()
+    torch.cuda.synchronize()
+    best = None
+    for _ in range(5):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        src.sum()
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b)
+        best = ms if best is None or ms < best else best
+    del src
+    return 4.0 * (1 << 30) / (best / 1e3) / 1e9
+
+
 def measured_copy_gbs(torch, dev):
     """Bandwidth of a plain 1 GiB device-to-device copy (read + write = 2 GiB moved), best of 5."""
     src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
@@ -269,7 +287,8 @@ def main():
     phases.mark("warm-up")
 
     copy_gbs = measured_copy_gbs(torch, dev)
-    log(f"[bench] 1 GiB device copy: {copy_gbs:.0f} GB/s")
+    read_gbs = measured_read_gbs(torch, dev)
+    log(f"[bench] 1 GiB device copy: {copy_gbs:.0f} GB/s; read-only pass over 4 GiB: {read_gbs:.0f} GB/s")
 
     # ---- the timed build: whole, hooks off ----
     profile_read(nv, reset=True, enable=0)
@@ -339,6 +358,7 @@ def main():
         achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
         traffic=traffic, traffic_detail=traffic_detail,
         copy_gbs_measured=copy_gbs, frac_of_measured_copy=achieved / copy_gbs if copy_gbs > 0 else None,
+        read_gbs_measured=read_gbs, frac_of_measured_read=achieved / read_gbs if read_gbs > 0 else None,
         avg_launch_ms=w_time / w_launch, algorithmic_bytes_per_launch=w_bytes / w_launch,
         launches_in_timed_build=int(sum(weights)),
         method=f"hooks are off in the timed build; the first {replay} batches of the tables each optimisation loop "
