@@ -935,3 +935,32 @@ def test_dense_seeding_ranked_by_leading_columns():
 
     say(f"  recall@10 all columns {recall(a):.3f}, 16 of 64 columns {recall(b):.3f}")
     assert recall(b) > recall(a) - 0.05
+
+
+def test_queues_beyond_64_kib_of_lds():
+    """Degree 256 with a build queue of 512: 2048 candidates per iteration, a visit queue of 768 and a visited
+    list of 3840 ids need about 90 KB of LDS per row, more than a kernel gets by default; the fused step, the
+    two-launch form and the queue kernels ask for it."""
+    say("queues that need more than 64 KiB of LDS")
+    from vectorlink_gpu import Queue
+    from vectorlink_gpu.ann import BEAM_TWO_LAUNCHES, closest_vectors, excluding_self
+
+    rng = np.random.default_rng(333)
+    n, dim, beam, bqf, pv = 1300, 8, 256, 2, 4
+    v = unit(rng, n, dim)
+    c = cfg(beam_size=beam, beam_queue_factor=bqf, parallel_visit_count=pv)
+    ql = beam * bqf
+    table = orc.generate_circulant_beams(n, orc.primes(ql))
+    d = orc.calculate_distances(v, table)
+    lo, hi = 100, 148
+    oq = orc.Queue(hi - lo, ql, ql + ql * pv)
+    oq.insert(table[lo:hi], d[lo:hi])
+    t_want = orc.closest_vectors(v[lo:hi], oq, v, table, c, orc.excluding_self(lo, hi))
+    gv, gb = dev(v), dev(table)
+    for flags in (0, BEAM_TWO_LAUNCHES):
+        gq = Queue(hi - lo, ql, ql + ql * pv)
+        gq.insert(gb[lo:hi], dev(d)[lo:hi])
+        t_got = closest_vectors(gv[lo:hi], gq, gv, gb, c, excluding_self(lo, hi), flags=flags)
+        assert t_got == t_want, flags
+        assert np.array_equal(host(gq.indices)[:, :ql], oq.indices[:, :ql]), flags
+        assert np.array_equal(bits(host(gq.distances)[:, :ql]), bits(oq.distances[:, :ql])), flags

@@ -837,10 +837,13 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
 template <int CPL, int LPR, int U, bool GENERIC>
 void launch_step(const StepArgs &s, int threads, size_t smem, hipStream_t st) {
     dim3 grid((unsigned)s.m.n_rows);
-    if (threads == 128)
+    if (threads == 128) {
+        if (vl_allow_lds(beam_step_kernel<CPL, LPR, U, GENERIC, 128>, smem) != hipSuccess) return;  // seen by the launch check
         hipLaunchKernelGGL((beam_step_kernel<CPL, LPR, U, GENERIC, 128>), grid, dim3(128), smem, st, s);
-    else
+    } else {
+        if (vl_allow_lds(beam_step_kernel<CPL, LPR, U, GENERIC, 256>, smem) != hipSuccess) return;
         hipLaunchKernelGGL((beam_step_kernel<CPL, LPR, U, GENERIC, 256>), grid, dim3(256), smem, st, s);
+    }
 }
 
 // VL_DIST_VARIANT (experiments only): 1 = two rows per load for rows of up to 512 bytes (32 lanes each) and
@@ -1037,7 +1040,8 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     const size_t smem = use_sort_merge
         ? (size_t)Pmax * 8 + (size_t)a.L * 4 + (size_t)a.E * 8 + (size_t)a.excl_cols * 4
         : (size_t)a.Pc * 24 + (size_t)(a.L + a.VL) * 8 + (size_t)a.E * 8 + (size_t)a.excl_cols * 4 + (size_t)a.m + 16;
-    VL_REQUIRE(smem <= 60 * 1024, "queues of this size need %zu bytes of LDS (limit 61440)", smem);
+    VL_REQUIRE(smem + 2048 <= kLdsPerCu, "queues of this size need %zu bytes of LDS (a compute unit has %zu)", smem,
+               kLdsPerCu);
 
     // VL_BEAM_FUSED=0 runs an iteration as two launches (expand, merge) instead of the fused step
     static const bool fused_env = [] {
@@ -1046,6 +1050,12 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     }();
     const bool use_fused = fused_env && !use_sort_merge && merge_threads != 64 && !(p->flags & VL_BEAM_TWO_LAUNCHES);
     VL_REQUIRE(!per_query || use_fused, "the per-query stop is only built into the fused step");
+    if (!use_fused) {
+        if (use_sort_merge) VL_HIP(vl_allow_lds(beam_merge_kernel, smem));
+        else if (merge_threads == 64) VL_HIP(vl_allow_lds(beam_merge2_kernel<64>, smem));
+        else if (merge_threads == 128) VL_HIP(vl_allow_lds(beam_merge2_kernel<128>, smem));
+        else VL_HIP(vl_allow_lds(beam_merge2_kernel<256>, smem));
+    }
     const bool aligned = (p->dim % 4 == 0) && (((uintptr_t)queries | (uintptr_t)vectors) % 16 == 0);
     StepArgs step;
     step.queries = queries; step.vectors = vectors; step.beams = beams; step.n_vectors = p->n_vectors;

@@ -27,7 +27,18 @@ constexpr int KT = 32;        // floats of the reduction dimension per stage
 constexpr int CH = KT / 4;    // 16-byte chunks per row and stage
 constexpr int TILE = 128 * KT;  // floats of one staged operand tile (16 KB)
 constexpr int LISTS_PER_STRIP = 4;  // two half-waves x two wave rows see the same query
-constexpr int64_t kResidentWorkgroups = 512;  // MI355X: 256 CUs, two workgroups of this kernel resident on each
+// workgroups of the tile kernel resident at once: two per compute unit (64 KB of LDS each), 256 CUs on an MI355X;
+// the count is read from the device on first use
+int64_t resident_workgroups() {
+    static const int64_t n = [] {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        return (int64_t)2 * cus;
+    }();
+    return n;
+}
 
 typedef __attribute__((address_space(3))) void lds_void;
 typedef __attribute__((address_space(1))) const void glb_void;
@@ -321,7 +332,7 @@ int knn_plan(int64_t n_queries, int64_t n_vectors, int64_t dim, int64_t k, KnnPl
     int64_t q_blocks = (n_queries + TQ - 1) / TQ;
     if (q_blocks < 1) q_blocks = 1;
     // The vector set is cut into at most 64 strips of whole tiles; q_blocks * strips workgroups
-    // share kResidentWorkgroups slots (256 CUs x 2 resident workgroups each), so the run lasts
+    // share resident_workgroups() slots (two per compute unit), so the run lasts
     // ceil(workgroups / slots) strips' worth of tiles.  Take the strip count with the shortest
     // run; a strip more costs a sixteenth of a tile (wider merge afterwards).
     const int64_t tiles = (n_vectors + TV - 1) / TV;
@@ -330,7 +341,7 @@ int knn_plan(int64_t n_queries, int64_t n_vectors, int64_t dim, int64_t k, KnnPl
         int64_t len_t = (tiles + s - 1) / s;
         int64_t s2 = (tiles + len_t - 1) / len_t;
         if (s2 != s) continue;
-        int64_t rounds = (q_blocks * s + kResidentWorkgroups - 1) / kResidentWorkgroups;
+        int64_t rounds = (q_blocks * s + resident_workgroups() - 1) / resident_workgroups();
         int64_t cost = rounds * len_t * 16 + s;
         if (best_cost < 0 || cost < best_cost) {
             best_cost = cost;

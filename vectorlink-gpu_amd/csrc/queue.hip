@@ -139,8 +139,9 @@ int launch_row_kernel(RowArgs a, hipStream_t st) {
     a.P = vl_next_pow2(a.cols);
     if (a.P < 2) a.P = 2;
     size_t smem = (size_t)a.P * 8 + (size_t)a.P * 4 + (size_t)(a.excl_cols > 0 ? a.excl_cols : 0) * 4;
-    VL_REQUIRE(smem <= 60 * 1024, "row of %d slots with %d exclusions needs %zu bytes of LDS (limit 61440)", a.cols,
-               a.excl_cols, smem);
+    VL_REQUIRE(smem + 2048 <= kLdsPerCu, "row of %d slots with %d exclusions needs %zu bytes of LDS (a compute unit has %zu)",
+               a.cols, a.excl_cols, smem, kLdsPerCu);
+    VL_HIP(vl_allow_lds(queue_row_kernel<MODE>, smem));
     for (a.row0 = 0; a.row0 < a.rows; a.row0 += kMaxBlocks) {
         int64_t rows = a.rows - a.row0 < kMaxBlocks ? a.rows - a.row0 : kMaxBlocks;
         hipLaunchKernelGGL((queue_row_kernel<MODE>), dim3((unsigned)rows), dim3(kQueueThreads), smem, st, a);

@@ -52,6 +52,18 @@ static inline unsigned vl_grid_for(int64_t n, int per_block) {
     return (unsigned)(b < 1 ? 1 : (b > kMaxBlocks ? kMaxBlocks : b));
 }
 
+// ---- LDS ---------------------------------------------------------------------
+// A gfx950 compute unit has 160 KiB of LDS and a workgroup may take all of it, but a launch that asks for
+// more dynamic LDS than the 64 KiB every kernel is allowed by default has to raise that kernel's limit first.
+constexpr size_t kLdsDefault = 64 * 1024;
+constexpr size_t kLdsPerCu = 160 * 1024;
+template <class Kernel>
+static inline hipError_t vl_allow_lds(Kernel kernel, size_t smem) {
+    if (smem + 1024 <= kLdsDefault) return hipSuccess;  // 1 KiB of slack for the kernels' static LDS
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)smem);
+}
+
 // ---- sort keys -------------------------------------------------------------
 // A queue slot is ordered by (distance asc, id asc).  The 64-bit key holds an
 // order-preserving image of the float in the high word and the id in the low

@@ -70,6 +70,30 @@ def _workspace(device) -> _Workspace:
     return ws
 
 
+def release_workspaces() -> None:
+    """Drop the scratch memory kept for beam searches (one block per device and stream, sized by the largest
+    batch seen; several GB after a large build).  The next search allocates what it needs again."""
+    with _WORKSPACES_LOCK:
+        for ws in _WORKSPACES.values():
+            with ws.lock:
+                ws.tensor = None
+
+
+_BUILD_STREAMS: Dict[str, list] = {}
+
+
+def _build_streams(device, lanes: int) -> list:
+    """The side streams every build on `device` shares (each stream owns a beam-search workspace, so builds
+    must not create streams of their own every time)."""
+    dev = torch.device(device)
+    index = dev.index if dev.index is not None else torch.cuda.current_device()
+    with _WORKSPACES_LOCK:
+        streams = _BUILD_STREAMS.setdefault(f"cuda:{index}", [])
+        while len(streams) < lanes:
+            streams.append(torch.cuda.Stream(device=index))
+        return streams[:lanes]
+
+
 def closest_vectors_stepwise(query_vecs: Tensor, search_queue: Queue, vectors: Tensor, beams: Tensor, config: Dict,
                              exclude: Optional[Tensor] = None) -> int:
     """The loop of ann.py:38-93 statement by statement on the single-purpose
@@ -252,8 +276,7 @@ class GraphBuild:
         (start, result) in the order of `starts`."""
         from concurrent.futures import ThreadPoolExecutor
 
-        if self._streams is None or len(self._streams) < lanes:
-            self._streams = [torch.cuda.Stream(device=device) for _ in range(lanes)]
+        self._streams = _build_streams(device, lanes)
         with ThreadPoolExecutor(max_workers=lanes) as pool:
             pending = []
             for k, start in enumerate(starts):
