@@ -396,6 +396,7 @@ def main():
         flops = 2.0 * qdev.shape[0] * n * dim
         result["exact_knn"] = dict(seconds=t_knn, tflops=flops / t_knn / 1e12, peak_tflops=MFMA_FP32_PEAK,
                                    frac=flops / t_knn / 1e12 / MFMA_FP32_PEAK, bound="mfma")
+        log(f"[bench] exact kNN: {result['exact_knn']}")
 
         def one_search(qs, seeding, mode):
             ann.search(qdev[:256].contiguous(), queue_size=qs, seeding=seeding, stop=mode)  # warm this shape
@@ -404,7 +405,9 @@ def main():
             res = ann.search(qdev, queue_size=qs, seeding=seeding, stop=mode)
             torch.cuda.synchronize()
             dt = time.time() - t0
-            return dict(queue=qs, qps=qdev.shape[0] / dt, recall_at_10=recall_at(res.indices[:, :10], truth))
+            r = dict(queue=qs, qps=qdev.shape[0] / dt, recall_at_10=recall_at(res.indices[:, :10], truth))
+            log(f"[bench] search: {seeding} seeds, {mode} stop, {r}")   # a line per setting: long legs stay audible
+            return r
 
         def sweep_search(seeding, mode):
             sweep, chosen = [], None

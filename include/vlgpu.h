@@ -295,6 +295,16 @@ int vl_knn_exact(const float *queries, int64_t n_queries,
                  const float *vectors, int64_t n_vectors, int64_t dim, int64_t k,
                  int32_t *ids_out, float *dists_out,
                  void *workspace, int64_t workspace_bytes, void *stream);
+/* The same under a metric (VL_METRIC_*).  L2 distances are formed as
+ * |q|^2 + |v|^2 - 2 q.v from the tiles' dot products and clamped at 0: a
+ * distance much smaller than the squared lengths carries their rounding
+ * (about 1e-7 of |q|^2 + |v|^2), so near-ties may order differently from the
+ * gathered-distance kernels, which subtract first.  The workspace of
+ * vl_knn_workspace_bytes serves both metrics. */
+int vl_knn_exact_metric(const float *queries, int64_t n_queries,
+                        const float *vectors, int64_t n_vectors, int64_t dim, int64_t k,
+                        int32_t metric, int32_t *ids_out, float *dists_out,
+                        void *workspace, int64_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

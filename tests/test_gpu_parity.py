@@ -854,8 +854,49 @@ def test_l2_build_and_search_against_oracle():
     truth = np.argsort(d2, axis=1)[:, :10]
     rec = np.mean([len(set(a[:10].tolist()) & set(t.tolist())) / 10 for a, t in zip(host(got.indices), truth)])
     assert rec > 0.8
-    with pytest.raises(ValueError):
-        ann.search(dev(qv), seeding="dense")
+    # dense seeding and recall@k follow the metric: the seeds are the nearest entry points by L2
+    dense = ann.search(dev(qv), seeding="dense")
+    found = host(dense.indices)[:, :10]
+    rec_dense = np.mean([len(set(a.tolist()) & set(t.tolist())) / 10 for a, t in zip(found, truth)])
+    assert rec_dense > 0.8
+    assert abs(ann.recall_at_k(dev(qv), 10, seeding="dense") - rec_dense) < 1e-9
+
+
+@pytest.mark.parametrize("n,dim,nq,k", [(5000, 128, 300, 10), (3000, 768, 129, 10), (1000, 20, 7, 16), (700, 36, 260, 1),
+                                        (6000, 100, 50, 12), (90, 4, 3, 2), (20000, 64, 64, 10)])
+def test_knn_exact_l2(n, dim, nq, k):
+    """Rows of unequal length, so the L2 order differs from the cosine order; truth is a float64
+    brute force that subtracts first."""
+    say(f"knn_exact L2 n={n} dim={dim} nq={nq} k={k}")
+    from vectorlink_gpu.kernels import knn_exact
+
+    rng = np.random.default_rng(3 * n + dim)
+    v = (rng.standard_normal((n, dim)) * rng.uniform(0.5, 2.0, (n, 1))).astype(np.float32)
+    q = (rng.standard_normal((nq, dim)) * rng.uniform(0.5, 2.0, (nq, 1))).astype(np.float32)
+    q[0] = v[17]  # an exact hit
+    with orc.metric("l2"):
+        wi, wd = orc.knn_exact(q, v, k)
+    d2 = ((q[:, None, :].astype(np.float64) - v[None, :, :].astype(np.float64)) ** 2).sum(2) if n * nq * dim < 3e8 else None
+    if d2 is not None:  # the oracle against numpy
+        order = np.argsort(d2, axis=1, kind="stable")[:, :k]
+        assert np.array_equal(order, wi)
+    ci, _ = knn_exact(dev(q), dev(v), k)
+    gi, gd = knn_exact(dev(q), dev(v), k, metric="l2")
+    gi, gd = host(gi), host(gd)
+    assert not np.array_equal(host(ci), gi)  # the metric matters on these rows
+    # |q|^2 + |v|^2 - 2 q.v carries the rounding of the squared lengths
+    scale = (q.astype(np.float64) ** 2).sum(1)[:, None] + (v.astype(np.float64) ** 2).sum(1).max()
+    tol = 4e-6 * scale
+    assert (np.abs(gd - wd) <= tol).all()
+    assert gi[0, 0] == 17
+    assert (np.diff(gd, axis=1) >= 0).all()
+    mism = gi != wi
+    assert mism.mean() < 0.02
+    for r, c in zip(*np.nonzero(mism)):
+        d_true = ((q[r].astype(np.float64) - v[gi[r, c]]) ** 2).sum()
+        assert abs(d_true - wd[r, c]) <= 2 * tol[r, 0]
+    for r in range(nq):
+        assert len(set(gi[r].tolist())) == k
 
 
 def test_self_recall_with_a_sample_that_is_not_the_head_of_the_vectors():

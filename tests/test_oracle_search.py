@@ -122,6 +122,20 @@ def test_knn_exact_against_numpy():
     assert np.allclose(d, np.take_along_axis(full, want, 1))
 
 
+def test_knn_exact_l2_against_numpy():
+    """Rows of unequal length: the squared-distance order differs from the cosine order."""
+    rng = np.random.default_rng(14)
+    v = (rng.standard_normal((500, 20)) * rng.uniform(0.5, 2, (500, 1))).astype(np.float32)
+    q = (rng.standard_normal((9, 20)) * rng.uniform(0.5, 2, (9, 1))).astype(np.float32)
+    with orc.metric("l2"):
+        ids, d = orc.knn_exact(q, v, 10)
+    cos_ids, _ = orc.knn_exact(q, v, 10)
+    full = ((q[:, None, :].astype(np.float64) - v[None, :, :].astype(np.float64)) ** 2).sum(2)
+    want = np.argsort(full, axis=1, kind="stable")[:, :10]
+    assert np.array_equal(ids, want) and not np.array_equal(ids, cos_ids)
+    assert np.allclose(d, np.take_along_axis(full, want, 1))
+
+
 def recall_at_k(found, truth):
     hits = sum(len(set(f.tolist()) & set(t.tolist())) for f, t in zip(found, truth))
     return hits / truth.size

@@ -1,5 +1,5 @@
-// Exact k nearest neighbours by cosine distance on dense fp32 MFMA tiles for
-// gfx950.  The reference has no counterpart (its recall is self-recall@1,
+// Exact k nearest neighbours by cosine or squared Euclidean distance on dense
+// fp32 MFMA tiles for gfx950.  The reference has no counterpart (its recall is self-recall@1,
 // vectorlink_gpu/ann.py:235-259); this is the ground truth for recall@k and the
 // only contraction-shaped step of the path.
 //
@@ -93,13 +93,36 @@ __device__ __forceinline__ void stage_operand(const float *const (&p)[4], int kt
 }
 
 // distance above which a value cannot enter a list whose last key is `last`
-__device__ __forceinline__ float list_bound(uint64_t last) { return last == kPadKey ? 2.0f : vl_key_dist(last); }
+__device__ __forceinline__ float list_bound(uint64_t last) { return last == kPadKey ? VL_MAXFLOAT : vl_key_dist(last); }
 
-template <int KK>
+// squared lengths of rows, one wavefront per row (the L2 tiles add them to -2 q.v)
+__global__ __launch_bounds__(256) void row_norms_kernel(const float *__restrict__ rows, int64_t n, int dim,
+                                                        float *__restrict__ out) {
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= n) return;
+    const int lane = threadIdx.x & 63;
+    const float4 *src = reinterpret_cast<const float4 *>(rows + row * dim);
+    float s = 0.0f;
+    for (int c = lane; c < dim / 4; c += 64) {
+        float4 x = src[c];
+        s = fmaf(x.x, x.x, s);
+        s = fmaf(x.y, x.y, s);
+        s = fmaf(x.z, x.z, s);
+        s = fmaf(x.w, x.w, s);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+    if (lane == 0) out[row] = s;
+}
+
+// L2: distances are |q|^2 + |v|^2 - 2 q.v from the rows' squared lengths (q_norm, v_norm)
+template <int KK, bool L2>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void knn_tile_kernel(const float *__restrict__ queries, int64_t n_queries,
                                                       const float *__restrict__ vectors, int64_t n_vectors,
                                                       int dim, int64_t strip_len, int n_strips,
-                                                      int n_qblocks, int q_group, uint64_t *__restrict__ cand) {
+                                                      int n_qblocks, int q_group, uint64_t *__restrict__ cand,
+                                                      const float *__restrict__ q_norm,
+                                                      const float *__restrict__ v_norm) {
     // two buffers per operand as separate arrays: the compiler can then tell that the loads
     // landing in one buffer do not touch the one being read
     __shared__ __align__(16) float sV0[TILE];
@@ -146,7 +169,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int i = 0; i < KK; ++i) list[cb][i] = kPadKey;
     // A value can only matter if it is not above the KK-th best seen so far for its query; the
     // two half-waves hold lists of the same queries, so each uses the tighter of the two bounds.
-    float bound[2] = {2.0f, 2.0f};
+    float bound[2] = {VL_MAXFLOAT, VL_MAXFLOAT};
 
     const int half = lane >> 5;   // which k of an MFMA pair this lane feeds
     const int l32 = lane & 31;
@@ -163,6 +186,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const bool ragged = (dim % KT) != 0;
     const float *qp[4], *vp[4];
     duty_pointers(queries, q0, n_queries - 1, dim, wave, lane, qp);
+    float qn[2] = {0.0f, 0.0f};
+    if constexpr (L2) {
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) {
+            const int64_t q = q0 + 64 * wc + 32 * cb + l32;
+            qn[cb] = q_norm[q < n_queries ? q : n_queries - 1];
+        }
+    }
 
     if (v_begin < v_end) {
         duty_pointers(vectors, v_begin, v_end - 1, dim, wave, lane, vp);
@@ -266,19 +297,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int vbase = (int)vt + 64 * wr + 4 * half;
         const int vlimit = (int)v_end;
 #pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
+        for (int rb = 0; rb < 2; ++rb) {
+            float vn[16];
+            if constexpr (L2) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int v = vbase + (32 * rb + 8 * (r >> 2) + (r & 3));
+                    vn[r] = v_norm[v < vlimit ? v : vlimit - 1];
+                }
+            }
 #pragma unroll
             for (int cb = 0; cb < 2; ++cb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int v = vbase + (32 * rb + 8 * (r >> 2) + (r & 3));
-                    float d = (1.0f - acc[rb][cb][r]) * 0.5f;
-                    d = d < 0.0f ? 0.0f : (d > 1.0f ? 1.0f : d);
+                    float d;
+                    if constexpr (L2) {
+                        d = fmaxf(fmaf(-2.0f, acc[rb][cb][r], qn[cb] + vn[r]), 0.0f);
+                    } else {
+                        d = (1.0f - acc[rb][cb][r]) * 0.5f;
+                        d = d < 0.0f ? 0.0f : (d > 1.0f ? 1.0f : d);
+                    }
                     if (v < vlimit && !(d > bound[cb])) {
                         uint64_t nk = vl_make_key(v, d);
                         if (nk < list[cb][KK - 1]) list_insert<KK>(list[cb], nk);
                     }
                 }
+        }
 #pragma unroll
         for (int cb = 0; cb < 2; ++cb) {
             float own = list_bound(list[cb][KK - 1]);
@@ -321,6 +366,7 @@ struct KnnPlan {
     int n_strips;
     int64_t strip_len;
     int n_cand;
+    int64_t cand_bytes;  // per-lane candidate lists; the rows' squared lengths (L2) follow
     int64_t bytes;
 };
 
@@ -353,7 +399,8 @@ int knn_plan(int64_t n_queries, int64_t n_vectors, int64_t dim, int64_t k, KnnPl
     p->strip_len = len;
     p->list_len = list_length(k);
     p->n_cand = (int)(strips * LISTS_PER_STRIP * p->list_len);
-    p->bytes = (n_queries > 0 ? n_queries : 1) * (int64_t)p->n_cand * 8;
+    p->cand_bytes = (n_queries > 0 ? n_queries : 1) * (int64_t)p->n_cand * 8;
+    p->bytes = p->cand_bytes + ((n_queries + n_vectors) * 4 + 15) / 16 * 16;
     return VL_OK;
 }
 
@@ -368,6 +415,14 @@ VL_EXPORT int64_t vl_knn_workspace_bytes(int64_t n_queries, int64_t n_vectors, i
 VL_EXPORT int vl_knn_exact(const float *queries, int64_t n_queries, const float *vectors,
                            int64_t n_vectors, int64_t dim, int64_t k, int32_t *ids_out,
                            float *dists_out, void *workspace, int64_t workspace_bytes, void *stream) {
+    return vl_knn_exact_metric(queries, n_queries, vectors, n_vectors, dim, k, VL_METRIC_COSINE, ids_out, dists_out,
+                               workspace, workspace_bytes, stream);
+}
+
+VL_EXPORT int vl_knn_exact_metric(const float *queries, int64_t n_queries, const float *vectors,
+                                  int64_t n_vectors, int64_t dim, int64_t k, int32_t metric, int32_t *ids_out,
+                                  float *dists_out, void *workspace, int64_t workspace_bytes, void *stream) {
+    VL_REQUIRE(metric == VL_METRIC_COSINE || metric == VL_METRIC_L2, "unknown metric %d", (int)metric);
     KnnPlan p;
     int rc = knn_plan(n_queries, n_vectors, dim, k, &p);
     if (rc < 0) return rc;
@@ -388,9 +443,28 @@ VL_EXPORT int vl_knn_exact(const float *queries, int64_t n_queries, const float 
     q_group = q_group < 1 ? 1 : (q_group > 8 ? 8 : q_group);
     const int64_t blocks = (q_blocks * p.n_strips + 7) / 8 * 8;
     VL_REQUIRE(blocks <= kMaxBlocks * 4, "too many tiles for one call");
-#define VL_KNN_LAUNCH(KK)                                                                                      \
-    hipLaunchKernelGGL(knn_tile_kernel<KK>, dim3((unsigned)blocks), dim3(256), 0, st, queries, n_queries, vectors, \
-                       n_vectors, (int)dim, p.strip_len, p.n_strips, (int)q_blocks, (int)q_group, cand)
+    const bool l2 = metric == VL_METRIC_L2;
+    float *q_norm = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + p.cand_bytes);
+    float *v_norm = q_norm + n_queries;
+    if (l2) {
+        VL_REQUIRE((n_vectors + 3) / 4 <= kMaxBlocks * 4, "too many vectors for one call");
+        hipLaunchKernelGGL(row_norms_kernel, dim3((unsigned)((n_queries + 3) / 4)), dim3(256), 0, st, queries,
+                           n_queries, (int)dim, q_norm);
+        hipLaunchKernelGGL(row_norms_kernel, dim3((unsigned)((n_vectors + 3) / 4)), dim3(256), 0, st, vectors,
+                           n_vectors, (int)dim, v_norm);
+        VL_LAUNCH_CHECK("row_norms_kernel");
+    }
+#define VL_KNN_LAUNCH(KK)                                                                                     \
+    do {                                                                                                      \
+        if (l2)                                                                                               \
+            hipLaunchKernelGGL((knn_tile_kernel<KK, true>), dim3((unsigned)blocks), dim3(256), 0, st, queries, \
+                               n_queries, vectors, n_vectors, (int)dim, p.strip_len, p.n_strips, (int)q_blocks, \
+                               (int)q_group, cand, q_norm, v_norm);                                           \
+        else                                                                                                  \
+            hipLaunchKernelGGL((knn_tile_kernel<KK, false>), dim3((unsigned)blocks), dim3(256), 0, st, queries, \
+                               n_queries, vectors, n_vectors, (int)dim, p.strip_len, p.n_strips, (int)q_blocks, \
+                               (int)q_group, cand, nullptr, nullptr);                                         \
+    } while (0)
     switch (p.list_len) {
         case 1: VL_KNN_LAUNCH(1); break;
         case 4: VL_KNN_LAUNCH(4); break;

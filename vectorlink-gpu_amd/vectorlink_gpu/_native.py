@@ -59,6 +59,7 @@ _SIGNATURES = {
     "vl_optimize_graph": (C.c_int, [_ptr, _i64, _i64, _i64, _ptr, _ptr, _i64, _ptr]),
     "vl_knn_workspace_bytes": (C.c_int64, [_i64, _i64, _i64, _i64]),
     "vl_knn_exact": (C.c_int, [_ptr, _i64, _ptr, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr]),
+    "vl_knn_exact_metric": (C.c_int, [_ptr, _i64, _ptr, _i64, _i64, _i64, C.c_int32, _ptr, _ptr, _ptr, _i64, _ptr]),
     "vl_prune": (C.c_int, [_ptr, _ptr, _i64, _i64, _ptr, _ptr, _ptr]),
 }
 

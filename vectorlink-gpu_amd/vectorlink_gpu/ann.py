@@ -388,7 +388,7 @@ def dense_search_queue(vectors: Tensor, query_vectors: Tensor, config: Dict, ent
     k = min(DENSE_SEEDS, entry_ids.size(0), queue_size)
     cols = entry_vectors.size(1)
     ranked_by = query_vectors if cols == query_vectors.size(1) else query_vectors[:, :cols].contiguous()
-    (local, _) = knn_exact(ranked_by, entry_vectors, k)
+    (local, _) = knn_exact(ranked_by, entry_vectors, k, config.get("metric", "cosine"))
     seeds = entry_ids[local.long()].contiguous()
     d = query_cosine_distances(query_vectors, vectors, seeds, config.get("metric", "cosine"))
     queue.insert(seeds, d)
@@ -494,11 +494,10 @@ class ANN:
         concurrent_batches (an addition) is the number of batches of an optimisation loop
         that the build keeps in flight, each on its own stream and host thread; the
         graph does not depend on it.  metric is an addition too: "cosine" is the reference's distance; "l2" builds
-        and searches by squared Euclidean distance (rows need not be unit length;
-        the dense seeding and recall_at_k tiles are cosine only and refuse it)."""
+        and searches by squared Euclidean distance (rows need not be unit length);
+        dense seeding and recall_at_k follow the metric."""
         assert prune in (True, False, "rank")
         nv.metric_code(metric)
-        assert not (metric == "l2" and seeding == "dense"), "dense seeding is cosine only"
         assert vectors.dim() == 2 and vectors.dtype == torch.float32
         assert seeding in ("circulant", "dense")
         self.seeding = seeding
@@ -637,8 +636,6 @@ class ANN:
         query = query.contiguous()
         seeding = seeding or self.seeding
         assert seeding in ("circulant", "dense")
-        if seeding == "dense" and self.configuration.get("metric", "cosine") != "cosine":
-            raise ValueError("dense seeding ranks entry points by cosine distance; use circulant seeds with metric='l2'")
         if seeding == "dense":
             (entry_ids, entry_vectors) = self._entry_tables()
             search_queue = dense_search_queue(self.vectors, query, self.configuration, entry_ids, entry_vectors,
@@ -654,13 +651,11 @@ class ANN:
         """Share of the exact k nearest neighbours (brute force on MFMA tiles)
         that search() returns in its first k slots.  Not in the reference,
         whose recall() is self-recall@1."""
-        if self.configuration.get("metric", "cosine") != "cosine":
-            raise ValueError("the exact-kNN tiles are cosine only")
         if not query.is_cuda:
             query = query.to(self.vectors.device)
         query = query.contiguous()
         found = self.search(query, queue_size, seeding).indices[:, :k]
-        (truth, _) = knn_exact(query, self.vectors, k)
+        (truth, _) = knn_exact(query, self.vectors, k, self.configuration.get("metric", "cosine"))
         hits = (found.unsqueeze(2) == truth.unsqueeze(1)).any(dim=2).sum().item()
         return hits / truth.numel()
 

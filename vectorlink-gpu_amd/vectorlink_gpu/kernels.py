@@ -159,8 +159,8 @@ def queue_sort_(ids: Tensor, distances: Tensor):
     nv.check(nv.lib().vl_queue_sort(nv.ptr(ids), nv.ptr(distances), ids.size(0), ids.size(1), nv.stream()))
 
 
-def knn_exact(queries: Tensor, vectors: Tensor, k: int) -> Tuple[Tensor, Tensor]:
-    """Exact k nearest neighbours by cosine distance on dense fp32 MFMA tiles
+def knn_exact(queries: Tensor, vectors: Tensor, k: int, metric: str = "cosine") -> Tuple[Tensor, Tensor]:
+    """Exact k nearest neighbours under `metric` on dense fp32 MFMA tiles
     (no counterpart in the reference; ground truth for recall@k).  Returns
     (ids [Q, k] int32, distances [Q, k] float32) ordered by (distance, id)."""
     _check_f32(queries, "queries")
@@ -172,8 +172,9 @@ def knn_exact(queries: Tensor, vectors: Tensor, k: int) -> Tuple[Tensor, Tensor]
     ws = torch.empty(max(need, 16), dtype=torch.uint8, device=vectors.device)
     ids = torch.empty((nq, k), dtype=torch.int32, device=vectors.device)
     dists = torch.empty((nq, k), dtype=torch.float32, device=vectors.device)
-    nv.check(nv.lib().vl_knn_exact(nv.ptr(queries), nq, nv.ptr(vectors), vectors.size(0), dim, k, nv.ptr(ids),
-                                   nv.ptr(dists), nv.ptr(ws), ws.numel(), nv.stream()))
+    nv.check(nv.lib().vl_knn_exact_metric(nv.ptr(queries), nq, nv.ptr(vectors), vectors.size(0), dim, k,
+                                          nv.metric_code(metric), nv.ptr(ids), nv.ptr(dists), nv.ptr(ws), ws.numel(),
+                                          nv.stream()))
     return (ids, dists)
 
 
