@@ -240,6 +240,7 @@ def main():
     ap.add_argument("--n", type=int, default=None, help="override the number of vectors")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-search", action="store_true", help="skip the search leg")
+    ap.add_argument("--no-tuned", action="store_true", help="skip the sweep of search settings (search_tuned)")
     ap.add_argument("--cpu-rows", type=int, default=768)
     ap.add_argument("--loops", type=int, default=3, help="optimisation loops of the build (the reference's default is 3)")
     ap.add_argument("--concurrent-batches", type=int, default=4,
@@ -450,7 +451,7 @@ def main():
         # length, how often progress is checked, which stop): the fastest of them that still reaches recall@10 >= 0.95
         tuned = []
         keep = (ann.entry_points, ann.configuration["speculative_readahead"], ann.seed_dims)
-        for entry_points in (32_768, 16_384, 8_192, 4_096):
+        for entry_points in () if args.no_tuned else (32_768, 16_384, 8_192, 4_096):
             for seed_dims in (None, 256 if dim > 256 else None, 128 if dim > 128 else None):
                 if seed_dims is None and (entry_points, None) in {(t["entry_points"], t["seed_dims"]) for t in tuned}:
                     continue

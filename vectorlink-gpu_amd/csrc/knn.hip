@@ -45,14 +45,21 @@ typedef __attribute__((address_space(1))) const void glb_void;
 
 __device__ __align__(16) const float kZeroChunk[4] = {0.f, 0.f, 0.f, 0.f};
 
+// A lane's list of the KK best so far: distances ascending with their ids.  A lane meets its
+// candidates in ascending id order, so one that ties a kept distance belongs behind it: comparing
+// distances alone orders (distance, id) pairs correctly.  The new distance column is a median of
+// three per slot; ids follow the same comparisons.
 template <int KK>
-__device__ __forceinline__ void list_insert(uint64_t (&key)[KK], uint64_t nk) {
+__device__ __forceinline__ void list_insert(float (&kd)[KK], int32_t (&kid)[KK], float d, int32_t id) {
 #pragma unroll
     for (int i = KK - 1; i > 0; --i) {
-        if (nk < key[i - 1]) key[i] = key[i - 1];
-        else if (nk < key[i]) key[i] = nk;
+        const bool before_prev = d < kd[i - 1], before_this = d < kd[i];
+        kid[i] = before_prev ? kid[i - 1] : (before_this ? id : kid[i]);
+        kd[i] = __builtin_amdgcn_fmed3f(kd[i - 1], d, kd[i]);
     }
-    if (nk < key[0]) key[0] = nk;
+    const bool first = d < kd[0];
+    kid[0] = first ? id : kid[0];
+    kd[0] = first ? d : kd[0];
 }
 
 // Chunk c (16 bytes) of tile row r lives in slot r * CH + (c ^ swz(r)): sixteen consecutive
@@ -91,9 +98,6 @@ __device__ __forceinline__ void stage_operand(const float *const (&p)[4], int kt
         __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(tile + 8 * (4 * wave + i) * KT), 16, 0, 0);
     }
 }
-
-// distance above which a value cannot enter a list whose last key is `last`
-__device__ __forceinline__ float list_bound(uint64_t last) { return last == kPadKey ? VL_MAXFLOAT : vl_key_dist(last); }
 
 // squared lengths of rows, one wavefront per row (the L2 tiles add them to -2 q.v)
 __global__ __launch_bounds__(256) void row_norms_kernel(const float *__restrict__ rows, int64_t n, int dim,
@@ -162,14 +166,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int64_t v_begin = strip * strip_len;
     const int64_t v_end = min(n_vectors, v_begin + strip_len);
 
-    uint64_t list[2][KK];
+    float kd[2][KK];
+    int32_t kid[2][KK];
 #pragma unroll
     for (int cb = 0; cb < 2; ++cb)
 #pragma unroll
-        for (int i = 0; i < KK; ++i) list[cb][i] = kPadKey;
+        for (int i = 0; i < KK; ++i) {
+            kd[cb][i] = __builtin_inff();   // an empty slot
+            kid[cb][i] = VL_MAXINT;
+        }
     // A value can only matter if it is not above the KK-th best seen so far for its query; the
     // two half-waves hold lists of the same queries, so each uses the tighter of the two bounds.
-    float bound[2] = {VL_MAXFLOAT, VL_MAXFLOAT};
+    float bound[2] = {__builtin_inff(), __builtin_inff()};
 
     const int half = lane >> 5;   // which k of an MFMA pair this lane feeds
     const int l32 = lane & 31;
@@ -293,9 +301,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             if (kt + KT < dim) stage(std::integral_constant<int, 1>{}, vt, kt + KT, acc);
         }
         // fold the 128 x 128 distances into the lists; accumulator register r of this lane:
-        // vector row 8*(r/4) + 4*half + r%4, query column l32 (ids stay below 2^30)
+        // vector row 8*(r/4) + 4*half + r%4, query column l32 (ids stay below 2^30).
+        // Nearly every value is beyond the bound once the lists have warmed up, so a block of 16
+        // values is first tested as a whole with one comparison per value, and only a block in
+        // which some lane has a candidate goes through the exact test and the insertion.
         const int vbase = (int)vt + 64 * wr + 4 * half;
         const int vlimit = (int)v_end;
+        // cosine: distance <= bound exactly when the dot product is at least 1 - 2 bound; the
+        // margin covers the rounding of (1 - dot) / 2 for dot products in [-1, 1], and every
+        // value passes while the bound is 1 or more (distances are clamped to 1)
+        float thr[2];
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb)
+            thr[cb] = bound[cb] >= 1.0f ? -__builtin_inff() : fmaf(-2.0f, bound[cb], 1.0f) - 4e-7f;
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
             float vn[16];
@@ -306,27 +324,35 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     vn[r] = v_norm[v < vlimit ? v : vlimit - 1];
                 }
             }
+            auto distance = [&](int cb, int r) {
+                if constexpr (L2) return fmaxf(fmaf(-2.0f, acc[rb][cb][r], qn[cb] + vn[r]), 0.0f);
+                const float d = (1.0f - acc[rb][cb][r]) * 0.5f;
+                return d < 0.0f ? 0.0f : (d > 1.0f ? 1.0f : d);
+            };
 #pragma unroll
-            for (int cb = 0; cb < 2; ++cb)
+            for (int cb = 0; cb < 2; ++cb) {
+                uint64_t hit[16], any = 0;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const int v = vbase + (32 * rb + 8 * (r >> 2) + (r & 3));
-                    float d;
-                    if constexpr (L2) {
-                        d = fmaxf(fmaf(-2.0f, acc[rb][cb][r], qn[cb] + vn[r]), 0.0f);
-                    } else {
-                        d = (1.0f - acc[rb][cb][r]) * 0.5f;
-                        d = d < 0.0f ? 0.0f : (d > 1.0f ? 1.0f : d);
-                    }
-                    if (v < vlimit && !(d > bound[cb])) {
-                        uint64_t nk = vl_make_key(v, d);
-                        if (nk < list[cb][KK - 1]) list_insert<KK>(list[cb], nk);
-                    }
+                    bool maybe;
+                    if constexpr (L2) maybe = !(distance(cb, r) > bound[cb]);
+                    else maybe = acc[rb][cb][r] >= thr[cb];
+                    hit[r] = __builtin_amdgcn_ballot_w64(maybe);
+                    any |= hit[r];
                 }
+                if (any == 0) continue;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    if (hit[r] == 0) continue;
+                    const int v = vbase + (32 * rb + 8 * (r >> 2) + (r & 3));
+                    const float d = distance(cb, r);
+                    if (v < vlimit && !(d > bound[cb]) && d < kd[cb][KK - 1]) list_insert<KK>(kd[cb], kid[cb], d, v);
+                }
+            }
         }
 #pragma unroll
         for (int cb = 0; cb < 2; ++cb) {
-            float own = list_bound(list[cb][KK - 1]);
+            const float own = kd[cb][KK - 1];
             bound[cb] = fminf(own, __shfl_xor(own, 32));
         }
     }
@@ -338,7 +364,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if (q < n_queries) {
             uint64_t *dst = cand + ((q * n_strips + strip) * LISTS_PER_STRIP + (wr * 2 + half)) * KK;
 #pragma unroll
-            for (int i = 0; i < KK; ++i) dst[i] = list[cb][i];
+            for (int i = 0; i < KK; ++i) dst[i] = kid[cb][i] == VL_MAXINT ? kPadKey : vl_make_key(kid[cb][i], kd[cb][i]);
         }
     }
 }
