@@ -399,7 +399,7 @@ def main():
                                    frac=flops / t_knn / 1e12 / MFMA_FP32_PEAK, bound="mfma")
         log(f"[bench] exact kNN: {result['exact_knn']}")
 
-        def one_search(qs, seeding, mode):
+        def one_search(qs, seeding, mode, quiet=False):
             ann.search(qdev[:256].contiguous(), queue_size=qs, seeding=seeding, stop=mode)  # warm this shape
             torch.cuda.synchronize()
             t0 = time.time()
@@ -407,7 +407,8 @@ def main():
             torch.cuda.synchronize()
             dt = time.time() - t0
             r = dict(queue=qs, qps=qdev.shape[0] / dt, recall_at_10=recall_at(res.indices[:, :10], truth))
-            log(f"[bench] search: {seeding} seeds, {mode} stop, {r}")   # a line per setting: long legs stay audible
+            if not quiet:
+                log(f"[bench] search: {seeding} seeds, {mode} stop, {r}")   # a line per setting: long legs stay audible
             return r
 
         def sweep_search(seeding, mode):
@@ -450,21 +451,29 @@ def main():
         # the same graph searched with other settings of the additions (entry points of the dense seeding, queue
         # length, how often progress is checked, which stop): the fastest of them that still reaches recall@10 >= 0.95
         tuned = []
-        keep = (ann.entry_points, ann.configuration["speculative_readahead"], ann.seed_dims)
-        for entry_points in () if args.no_tuned else (32_768, 16_384, 8_192, 4_096):
+        keep = (ann.entry_points, ann.configuration["speculative_readahead"], ann.seed_dims,
+                ann.configuration["parallel_visit_count"])
+        seen_settings = set()
+        for entry_points in () if args.no_tuned else (32_768, 16_384, 8_192):
             for seed_dims in (None, 256 if dim > 256 else None, 128 if dim > 128 else None):
-                if seed_dims is None and (entry_points, None) in {(t["entry_points"], t["seed_dims"]) for t in tuned}:
+                if (entry_points, seed_dims) in seen_settings:
                     continue
-                for readahead in (2, 5):
-                    for qs in (10, 16, 32):
-                        for mode in ("batch", "per_query"):
-                            ann.entry_points, ann.seed_dims, ann._entry = entry_points, seed_dims, None
-                            ann.configuration["speculative_readahead"] = readahead
-                            r = one_search(qs, "dense", mode)
-                            r.update(entry_points=entry_points, seed_dims=seed_dims, speculative_readahead=readahead,
-                                     stop=mode)
-                            tuned.append(r)
-        (ann.entry_points, ann.configuration["speculative_readahead"], ann.seed_dims), ann._entry = keep, None
+                seen_settings.add((entry_points, seed_dims))
+                for visit in (2, 3, 4):
+                    for readahead in (1, 2, 5):
+                        for qs in (10, 16):
+                            for mode in ("batch", "per_query"):
+                                ann.entry_points, ann.seed_dims, ann._entry = entry_points, seed_dims, None
+                                ann.configuration["speculative_readahead"] = readahead
+                                ann.configuration["parallel_visit_count"] = visit
+                                r = one_search(qs, "dense", mode, quiet=True)
+                                r.update(entry_points=entry_points, seed_dims=seed_dims, parallel_visit_count=visit,
+                                         speculative_readahead=readahead, stop=mode)
+                                tuned.append(r)
+            log(f"[bench] search sweep: {len(tuned)} settings tried")
+        (ann.entry_points, ann.configuration["speculative_readahead"], ann.seed_dims,
+         ann.configuration["parallel_visit_count"]) = keep
+        ann._entry = None
         ok = [r for r in tuned if r["recall_at_10"] >= 0.95]
         result["search_tuned"] = dict(tried=tuned, best=max(ok, key=lambda r: r["qps"]) if ok else None,
                                       best_with_the_reference_stop=max(

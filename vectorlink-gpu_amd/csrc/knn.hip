@@ -369,18 +369,60 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
-__global__ __launch_bounds__(kQueueThreads) void knn_merge_kernel(const uint64_t *__restrict__ cand, int n_cand, int P,
-                                                                 int k, int32_t *ids_out, float *d_out, int64_t q0) {
-    extern __shared__ __align__(16) unsigned char smem[];
-    uint64_t *keys = reinterpret_cast<uint64_t *>(smem);
-    const int64_t q = q0 + blockIdx.x;
-    for (int i = threadIdx.x; i < P; i += blockDim.x) keys[i] = i < n_cand ? cand[q * n_cand + i] : kPadKey;
-    block_bitonic_sort(keys, P);
-    for (int i = threadIdx.x; i < k; i += blockDim.x) {
-        uint64_t key = keys[i];
-        bool real = key != kPadKey;
-        ids_out[q * k + i] = real ? vl_key_id(key) : VL_MAXINT;
-        d_out[q * k + i] = real ? vl_key_dist(key) : VL_MAXFLOAT;
+// A query's candidates are n_lists lists of KK keys, each sorted, and no id is in two of them.  One
+// wavefront merges them as a tournament: a lane keeps the heads of its lists (lane, lane + 64, ...)
+// and the key behind each head; the smallest head of the wavefront is the next result and the lane
+// that held it moves on in that list.  Only the heads and the few keys behind a winner are read.
+constexpr int kSelectLists = 4;  // lists per lane: 64 strips x 4 lists at most
+
+__global__ __launch_bounds__(256) void knn_select_kernel(const uint64_t *__restrict__ cand, int n_lists, int KK, int k,
+                                                         int32_t *__restrict__ ids_out, float *__restrict__ d_out,
+                                                         int64_t n_queries) {
+    const int64_t q = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (q >= n_queries) return;  // the whole wavefront leaves
+    const int lane = threadIdx.x & 63;
+    const uint64_t *base = cand + q * n_lists * KK;
+    uint64_t head[kSelectLists], next[kSelectLists];
+    int pos[kSelectLists];
+#pragma unroll
+    for (int j = 0; j < kSelectLists; ++j) {
+        const int list = lane + 64 * j;
+        head[j] = list < n_lists ? base[(int64_t)list * KK] : kPadKey;
+        next[j] = list < n_lists && KK > 1 ? base[(int64_t)list * KK + 1] : kPadKey;
+        pos[j] = 0;
+    }
+    uint64_t result = kPadKey;
+    for (int i = 0; i < k; ++i) {
+        uint64_t mine = head[0];
+        int which = 0;
+#pragma unroll
+        for (int j = 1; j < kSelectLists; ++j)
+            if (head[j] < mine) {
+                mine = head[j];
+                which = j;
+            }
+        uint64_t best = mine;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const uint64_t other = __shfl_xor(best, o);
+            best = other < best ? other : best;
+        }
+        if (best == kPadKey) break;  // fewer than k candidates in all
+        if (lane == i) result = best;
+        if (mine == best) {  // keys are unique: one lane moves on, in one list
+#pragma unroll
+            for (int j = 0; j < kSelectLists; ++j)
+                if (j == which) {
+                    ++pos[j];
+                    head[j] = next[j];
+                    next[j] = pos[j] + 1 < KK ? base[(int64_t)(lane + 64 * j) * KK + pos[j] + 1] : kPadKey;
+                }
+        }
+    }
+    if (lane < k) {
+        const bool real = result != kPadKey;
+        ids_out[q * k + lane] = real ? vl_key_id(result) : VL_MAXINT;
+        d_out[q * k + lane] = real ? vl_key_dist(result) : VL_MAXFLOAT;
     }
 }
 
@@ -501,12 +543,10 @@ VL_EXPORT int vl_knn_exact_metric(const float *queries, int64_t n_queries, const
     }
 #undef VL_KNN_LAUNCH
     VL_LAUNCH_CHECK("knn_tile_kernel");
-    int P = vl_next_pow2(p.n_cand);
-    for (int64_t q0 = 0; q0 < n_queries; q0 += kMaxBlocks) {
-        int64_t rows = n_queries - q0 < kMaxBlocks ? n_queries - q0 : kMaxBlocks;
-        hipLaunchKernelGGL(knn_merge_kernel, dim3((unsigned)rows), dim3(kQueueThreads), (size_t)P * 8, st, cand,
-                           p.n_cand, P, (int)k, ids_out, dists_out, q0);
-    }
-    VL_LAUNCH_CHECK("knn_merge_kernel");
+    const int n_lists = p.n_strips * LISTS_PER_STRIP;
+    VL_REQUIRE(n_lists <= 64 * kSelectLists, "too many candidate lists per query");
+    hipLaunchKernelGGL(knn_select_kernel, dim3((unsigned)((n_queries + 3) / 4)), dim3(256), 0, st, cand, n_lists,
+                       p.list_len, (int)k, ids_out, dists_out, n_queries);
+    VL_LAUNCH_CHECK("knn_select_kernel");
     return VL_OK;
 }
