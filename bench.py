@@ -413,7 +413,7 @@ def main():
 
         def sweep_search(seeding, mode):
             sweep, chosen = [], None
-            for qs in (16, 32, 64, 96, 128, 192, 256):
+            for qs in (10, 16, 32, 64, 96, 128, 192, 256):
                 sweep.append(one_search(qs, seeding, mode))
                 if chosen is None and sweep[-1]["recall_at_10"] >= 0.95:
                     chosen = sweep[-1]

@@ -926,7 +926,10 @@ int beam_layout(const vl_beam_params *p, BeamLayout *l, bool lean = false) {
         const char *e = getenv("VL_BEAM_MEMO");
         return e ? atoi(e) : -1;
     }();
-    int slots = vl_next_pow2(128 * l->m);
+    // ... and no more than 512 per slot of the search queue: a search with a short queue ends after few
+    // iterations, fills little of a large table and would pay for clearing it on every call
+    int64_t want = 128 * l->m < 512 * p->queue_length ? 128 * l->m : 512 * p->queue_length;
+    int slots = vl_next_pow2(want > 65536 ? 65536 : want);
     if (slots < 1024) slots = 1024;
     if (slots > 65536) slots = 65536;
     while (slots > 1024 && p->n_rows * (int64_t)slots * 8 > (8ll << 30)) slots >>= 1;
@@ -1030,12 +1033,14 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     }();
     const bool use_sort_merge = sort_merge_env || (p->flags & VL_BEAM_SORT_MERGE);
     // threads per row of the merge step: small rows are latency bound and do better with
-    // more rows in flight per CU (measured: 128 wins at m=256, E=480; 256 wins at m=512, E=960)
+    // more rows in flight per CU (measured: 128 wins at m=256, E=480 and at m=128, E=960; 256 wins at
+    // m=512, E=960)
     static const int merge_threads_env = [] {
         const char *e = getenv("VL_BEAM_MERGE_THREADS");
         return e ? atoi(e) : 0;
     }();
-    const int merge_threads = merge_threads_env ? merge_threads_env : ((l.m + l.E + l.VL + p->queue_length) <= 1024 ? 128 : 256);
+    const int merge_threads = merge_threads_env ? merge_threads_env
+                              : ((l.m <= 128 || (l.m + l.E + l.VL + p->queue_length) <= 1024) ? 128 : 256);
     const int Pmax = a.Ps > a.Pv ? a.Ps : a.Pv;
     const size_t smem = use_sort_merge
         ? (size_t)Pmax * 8 + (size_t)a.L * 4 + (size_t)a.E * 8 + (size_t)a.excl_cols * 4
