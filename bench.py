@@ -241,6 +241,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-search", action="store_true", help="skip the search leg")
     ap.add_argument("--no-tuned", action="store_true", help="skip the sweep of search settings (search_tuned)")
+    ap.add_argument("--knn-only", action="store_true",
+                    help="only the dense MFMA tiles on this workload's vectors (exact kNN of the queries, and the "
+                         "seeding pass over 32,768 entry points); prints their figures as the JSON line")
     ap.add_argument("--cpu-rows", type=int, default=768)
     ap.add_argument("--loops", type=int, default=3, help="optimisation loops of the build (the reference's default is 3)")
     ap.add_argument("--concurrent-batches", type=int, default=4,
@@ -275,6 +278,30 @@ def main():
     vectors = base.to(dev)
     qdev = queries.to(dev)
     torch.cuda.synchronize()
+
+    if args.knn_only:
+        out = {"metric": "dense distance tiles (fp32 MFMA), TFLOP/s", "unit": "TFLOP/s", "n_gpus": 1,
+               "higher_is_better": True, "dtype": "f32", "data": "synthetic",
+               "config": {"workload": args.workload, "n": n, "dim": dim, "queries": int(qdev.shape[0])}}
+        from vectorlink_gpu.ann import entry_point_ids
+        entries = vectors[entry_point_ids(n, 32_768, dev).long()].contiguous()
+        for (name, table, k) in (("exact_knn", vectors, 10), ("seeding_tiles", entries, 16)):
+            knn_exact(qdev, table, k)
+            torch.cuda.synchronize()
+            reps = max(1, args.steps // 4)
+            t0 = time.time()
+            for _ in range(reps):
+                knn_exact(qdev, table, k)
+            torch.cuda.synchronize()
+            dt = (time.time() - t0) / reps
+            flops = 2.0 * qdev.shape[0] * table.shape[0] * dim
+            out[name] = dict(bound="mfma", vectors=int(table.shape[0]), k=k, seconds=dt, tflops=flops / dt / 1e12,
+                             peak_tflops=MFMA_FP32_PEAK, frac=flops / dt / 1e12 / MFMA_FP32_PEAK, calls=reps + 1)
+        out["value"] = out["exact_knn"]["tflops"]
+        out["roofline"] = dict(bound="mfma", achieved=out["exact_knn"]["tflops"], peak=MFMA_FP32_PEAK, unit="TFLOP/s",
+                               frac=out["exact_knn"]["frac"], traffic=None)
+        print(json.dumps(out))
+        return
 
     phases = Phases()
     # warm-up: a small separate build (kernels loaded, allocator primed)
