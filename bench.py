@@ -56,9 +56,10 @@ def log(*a):
 
 
 def profile_read(nv, reset=True, enable=1):
-    out = (ctypes.c_double * 8)()
+    out = (ctypes.c_double * 9)()
     nv.lib().vl_beam_profile(enable, 1 if reset else 0, out)
-    keys = ("expand_ms", "merge_ms", "expand_launches", "merge_launches", "evals", "rows", "iterations", "wanted")
+    keys = ("expand_ms", "merge_ms", "expand_launches", "merge_launches", "evals", "rows", "iterations", "wanted",
+            "sketched")
     return dict(zip(keys, list(out)))
 
 

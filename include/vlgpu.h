@@ -202,6 +202,10 @@ typedef struct vl_beam_params {
  * against, the CPU model closest_vectors_per_query of the test oracle.  Fused
  * step only. */
 #define VL_BEAM_PER_QUERY_STOP 4
+/* Same loop, same result, without the per-row cache of already evaluated
+ * (id, distance) pairs: the workspace shrinks by the cache's table and every
+ * candidate distance is evaluated when it is asked for. */
+#define VL_BEAM_NO_CACHE 8
 
 int64_t vl_beam_workspace_bytes(const vl_beam_params *p);
 
@@ -218,6 +222,45 @@ int64_t vl_closest_vectors(const vl_beam_params *p,
                            const int32_t *exclude,
                            void *workspace, int64_t workspace_bytes,
                            void *stream);
+
+/* ---- 8-bit sketch of the vector table (no counterpart in the reference) --
+ *
+ * The reference evaluates every candidate distance of an iteration in full
+ * (cuda_search_from_seeds_kernel, kernels.py:204-257) although a row keeps a
+ * handful of its hundreds of candidates.  A sketch row holds the vector rounded
+ * to 8 bits per element with one scale per row (dim bytes, padded to a multiple
+ * of 16) and a 16-byte tail: float scale, float bound on the 2-norm of what the
+ * rounding moved, float bound on the row's 2-norm, float 0.  With it a dot
+ * product is known to within ||q|| x that bound (Cauchy-Schwarz) from a quarter
+ * of the bytes.  vl_closest_vectors_with_sketch uses those bounds ONLY to decide
+ * which candidate rows to fetch: a candidate whose lower bound is above the last
+ * slot of the search queue and, when it is unvisited, above the last live slot
+ * of the visit queue and above the parallel_visit_count-th smallest upper bound
+ * beyond it, cannot enter either queue and is dropped; every other candidate is
+ * evaluated exactly.  Queues are bit-identical to vl_closest_vectors'. */
+
+/* Bytes per sketch row for vectors of `dim` columns: 16 * ceil(dim / 16) + 16. */
+int64_t vl_sketch_row_bytes(int64_t dim);
+
+/* Fills table[n_vectors, vl_sketch_row_bytes(dim)] (16-byte aligned) from
+ * vectors[n_vectors, dim].  A row holding a NaN or an infinity gets an infinite
+ * bound: its candidates are always evaluated exactly. */
+int vl_sketch_build(const float *vectors, int64_t n_vectors, int64_t dim,
+                    uint8_t *table, void *stream);
+
+/* vl_closest_vectors with the sketch of `vectors` (NULL: exactly
+ * vl_closest_vectors).  Same arguments, same result, same return value.  The
+ * sketch serves the fused step under the cosine metric for 16-byte aligned rows
+ * of up to 2048 columns; other calls ignore it.  Each row decides for itself:
+ * rows whose candidates mostly repeat keep the distance cache instead. */
+int64_t vl_closest_vectors_with_sketch(const vl_beam_params *p,
+                                       const float *queries, const float *vectors,
+                                       const uint8_t *sketch,
+                                       const int32_t *beams,
+                                       int32_t *q_ids, float *q_dists,
+                                       const int32_t *exclude,
+                                       void *workspace, int64_t workspace_bytes,
+                                       void *stream);
 
 /* vl_closest_vectors for callers that cannot allocate or wait: code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has
@@ -249,11 +292,12 @@ int vl_closest_vectors_noalloc(const vl_beam_params *p,
 
 /* Per-kernel timing of vl_closest_vectors (no counterpart in the reference,
  * whose log.py:7-17 times whole calls): with enable != 0 every expand / merge
- * launch is bracketed by HIP events on the caller's stream.  out (8 doubles,
+ * launch is bracketed by HIP events on the caller's stream.  out (9 doubles,
  * may be NULL) receives the sums since the last reset: expand ms, merge ms,
  * expand launches, merge launches, candidate rows fetched, query rows,
  * iterations, candidate distances asked for (fetched + served by the per-row
- * cache of already evaluated pairs).  The sums are kept under a mutex, so
+ * cache of already evaluated pairs), candidate rows looked at through the
+ * sketch.  The sums are kept under a mutex, so
  * profiled calls from several host threads add up without tearing. */
 int vl_beam_profile(int enable, int reset, double *out);
 

@@ -1005,3 +1005,125 @@ def test_queues_beyond_64_kib_of_lds():
         assert t_got == t_want, flags
         assert np.array_equal(host(gq.indices)[:, :ql], oq.indices[:, :ql]), flags
         assert np.array_equal(bits(host(gq.distances)[:, :ql]), bits(oq.distances[:, :ql])), flags
+
+
+# ---------------------------------------------------------------- 8-bit sketch
+@pytest.mark.parametrize("dim", [4, 20, 64, 100, 128, 384, 768, 1000, 1536, 2048])
+def test_sketch_rows_bound_every_dot_product(dim):
+    """build_sketch: the bytes are the row rounded to 8 bits under the row's own scale, and the tail's two
+    bounds hold against float64 - the 2-norm of what the rounding moved, and the row's 2-norm.  Then, for
+    random queries, |<q, v> - scale * <q, u - 128>| <= ||q|| * bound, which is what the search relies on."""
+    say(f"sketch rows dim={dim}")
+    from vectorlink_gpu.kernels import build_sketch, sketch_row_bytes
+
+    rng = np.random.default_rng(dim)
+    n = 300
+    v = unit(rng, n, dim)
+    v[1] = 0.0                               # an all-zero row
+    v[2] *= 37.5                             # not a unit row
+    v[3, ::2] = 0.0
+    v[4] = np.float32(1e-30) * v[4]          # tiny
+    if dim > 4:
+        v[5, 3] = np.nan                     # promises nothing
+        v[6, 1] = np.inf
+    rb = sketch_row_bytes(dim)
+    assert rb == 16 * ((dim + 15) // 16) + 16
+    t = host(build_sketch(dev(v)))
+    assert t.shape == (n, rb)
+    pad = rb - 16
+    u = t[:, :dim].astype(np.float64) - 128.0
+    tail = t[:, pad:].copy().view(np.float32)
+    scale, resid, norm = tail[:, 0].astype(np.float64), tail[:, 1].astype(np.float64), tail[:, 2].astype(np.float64)
+    assert np.all(t[:, dim:pad] == 128) and np.all(tail[:, 3] == 0)
+    bad = ~np.isfinite(v).all(axis=1)
+    assert np.all(np.isinf(resid[bad])) and np.all(np.isinf(norm[bad]))
+    ok = ~bad
+    v64 = v[ok].astype(np.float64)
+    assert np.all(np.abs(u[ok]) <= 127)
+    moved = np.linalg.norm(v64 - scale[ok, None] * u[ok], axis=1)
+    assert np.all(resid[ok] >= moved)
+    assert np.all(norm[ok] >= np.linalg.norm(v64, axis=1))
+    # tight: rounding moves an element by at most half a step, and the bounds are within 0.2 % of the truth
+    assert np.all(moved <= 0.5 * scale[ok] * np.sqrt(dim) * (1 + 1e-6) + 1e-30)
+    assert np.all(resid[ok] <= moved * 1.002 + 1e-17) and np.all(norm[ok] <= np.linalg.norm(v64, axis=1) * 1.002 + 1e-17)
+    mx = np.abs(v64).max(axis=1)
+    assert np.allclose(scale[ok], mx / 127.0, rtol=1e-6, atol=0)
+    q = unit(rng, 50, dim).astype(np.float64)
+    exact = q @ v64.T
+    approx = (q @ u[ok].T) * scale[ok][None, :]
+    assert np.all(np.abs(exact - approx) <= np.linalg.norm(q, axis=1)[:, None] * resid[ok][None, :] + 1e-12)
+
+
+SKETCH_CASES = [
+    # n, dim, beam, bqf, pv, vqf, ef, ra
+    (700, 16, 4, 2, 2, 3, 5, 5),       # one chunk per sketch row
+    (900, 64, 8, 2, 4, 3, 5, 5),
+    (1200, 100, 8, 2, 4, 3, 5, 5),     # a last chunk that is only partly data
+    (2000, 128, 32, 2, 4, 3, 5, 5),    # the 128-column benchmark shape
+    (1500, 256, 16, 2, 4, 3, 5, 5),
+    (1500, 384, 48, 2, 4, 3, 5, 5),
+    (1200, 512, 16, 2, 4, 3, 5, 5),
+    (2000, 768, 64, 2, 4, 3, 5, 5),    # the 768-column benchmark shape
+    (1200, 1024, 16, 2, 4, 3, 5, 5),
+    (800, 1280, 8, 2, 3, 3, 5, 2),
+    (1200, 1536, 24, 3, 4, 3, 5, 5),
+    (600, 1792, 8, 2, 4, 2, 2, 3),     # a visited list that runs full
+    (600, 2048, 8, 2, 9, 4, 2, 4),
+    (500, 2052, 8, 2, 4, 3, 5, 5),     # beyond the sketch's sizes: ignored
+    (500, 130, 8, 2, 4, 3, 5, 5),      # rows that are not 16-byte aligned: ignored
+]
+
+
+@pytest.mark.parametrize("n,dim,beam,bqf,pv,vqf,ef,ra", SKETCH_CASES)
+@pytest.mark.parametrize("cache", [False, True])
+def test_closest_vectors_with_sketch(n, dim, beam, bqf, pv, vqf, ef, ra, cache):
+    """The loop with the 8-bit sketch against the oracle: same iteration count, ids and distance bits.
+    Without the distance cache every row looks through the sketch from the first iteration; with it, rows
+    measure their share of cache hits first (random rows on a circulant graph: hardly any) and then switch.
+    The profiling counters show that the sketch was really used."""
+    say(f"closest_vectors with sketch n={n} dim={dim} beam={beam} cache={cache}")
+    import ctypes
+
+    from vectorlink_gpu import Queue
+    from vectorlink_gpu import _native as nv
+    from vectorlink_gpu.ann import BEAM_NO_CACHE, closest_vectors, excluding_self
+    from vectorlink_gpu.kernels import build_sketch
+
+    rng = np.random.default_rng(n + dim)
+    v = unit(rng, n, dim)
+    if dim >= 64:
+        v[5] = v[9]            # exact duplicate rows: ties ordered by id
+        v[11] *= 1.5           # a row that is not of unit length
+    c = cfg(beam_size=beam, beam_queue_factor=bqf, parallel_visit_count=pv, visit_queue_factor=vqf,
+            exclude_factor=ef, speculative_readahead=ra)
+    ql = beam * bqf
+    beams = orc.generate_circulant_beams(n, orc.primes(ql))
+    d = orc.calculate_distances(v, beams)
+    lo, hi = 0, min(n, 600)
+    oq = orc.Queue(hi - lo, ql, ql + ql * pv)
+    oq.insert(beams[lo:hi], d[lo:hi])
+    t_want = orc.closest_vectors(v[lo:hi], oq, v, beams, c, orc.excluding_self(lo, hi))
+
+    gv, gb = dev(v), dev(beams)
+    sk = build_sketch(gv)
+    gq = Queue(hi - lo, ql, ql + ql * pv)
+    gq.insert(gb[lo:hi], dev(d)[lo:hi])
+    out = (ctypes.c_double * 9)()
+    nv.lib().vl_beam_profile(1, 1, out)
+    try:
+        t_got = closest_vectors(gv[lo:hi], gq, gv, gb, c, excluding_self(lo, hi), flags=0 if cache else BEAM_NO_CACHE,
+                                sketch=sk)
+    finally:
+        nv.lib().vl_beam_profile(0, 1, out)
+    (fetched, wanted, sketched) = (out[4], out[7], out[8])
+    say(f"  iterations {t_got}, candidates {wanted:.0f}, through the sketch {sketched:.0f}, rows fetched {fetched:.0f}")
+    assert t_got == t_want
+    assert np.array_equal(host(gq.indices)[:, :ql], oq.indices[:, :ql])
+    assert np.array_equal(bits(host(gq.distances)[:, :ql]), bits(oq.distances[:, :ql]))
+    if dim % 4 == 0 and dim <= 2048:
+        if not cache:
+            assert sketched == wanted and fetched < 0.8 * wanted
+        elif t_got > 15:
+            assert sketched > 0 or fetched < 0.5 * wanted   # rows whose candidates repeat keep the cache instead
+    else:
+        assert sketched == 0

@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 OUT = os.path.join(HERE, "vectorlink_gpu", "libvlgpu.so")
 
-SOURCES = ["error.cpp", "dist.hip", "queue.hip", "prune.hip", "beam.hip", "knn.hip", "graphopt.hip"]
+SOURCES = ["error.cpp", "dist.hip", "queue.hip", "prune.hip", "beam.hip", "knn.hip", "graphopt.hip", "sketch.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",

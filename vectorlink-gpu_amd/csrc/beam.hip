@@ -20,6 +20,7 @@
 #include "beam_ctrl.h"
 #include "rowsort.h"
 #include "dist_device.h"
+#include "sketch_device.h"
 #include <stdlib.h>
 #include <mutex>
 
@@ -39,7 +40,7 @@ constexpr int kMaxVisit = 64;  // parallel_visit_count handled by one wavefront
 struct BeamProfile {
     int enabled = 0;
     double expand_ms = 0, merge_ms = 0;
-    int64_t expand_launches = 0, merge_launches = 0, evals = 0, rows = 0, iterations = 0, wanted = 0;
+    int64_t expand_launches = 0, merge_launches = 0, evals = 0, rows = 0, iterations = 0, wanted = 0, sketched = 0;
 };
 // The only mutable state of the library besides the thread-local error text.  A call
 // sums into a BeamProfile of its own and adds it here once, under the mutex, when it
@@ -116,11 +117,13 @@ __global__ __launch_bounds__(kQueueThreads) void beam_init_kernel(BeamCtrl *ctrl
         ctrl->stop = 0;
         ctrl->ended_after = 0;
         ctrl->first[0] = ctrl->first[1] = ctrl->first[2] = 0;
+        ctrl->cache_dropped = 0;
     }
     if (t < 64) ctrl->changed[t] = 0;
     if (t < kBeamStripes) {
         ctrl->evals[t] = 0;
         ctrl->wanted[t] = 0;
+        ctrl->sketched[t] = 0;
     }
     if (t < n_rows) {
         seen_count[t] = 0;
@@ -370,8 +373,16 @@ struct RowState {
 // written by the expand phase of the same workgroup), the loop state has been checked, and
 // the row's queues, visited list, popped ids and exclusions have been placed in LDS by
 // stage_row (the global reads were issued at the start of the kernel).
-template <int THREADS, bool FUSED>
-__device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *smem, RowState pre = RowState{0, 0}) {
+// refine (fused step only): called once the visited list is current and before the candidates are
+// looked at, with the last slots of both queues; it may replace candidate distances that are only known
+// as bounds by exact ones and drop candidates that provably cannot enter a queue.
+struct NoRefine {
+    __device__ __forceinline__ void operator()(const int32_t *, int, bool, uint64_t, uint64_t, uint8_t *, uint64_t *) const {}
+};
+
+template <int THREADS, bool FUSED, class Refine = NoRefine>
+__device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *smem, RowState pre = RowState{0, 0},
+                                          Refine refine = Refine()) {
     const int Pc = a.Pc;
     uint64_t *raw = reinterpret_cast<uint64_t *>(smem);  // candidate keys as they arrive
     uint64_t *uk = raw + Pc;                             // the candidates that can matter, then sorted
@@ -409,9 +420,6 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
     // the ids popped at the start of this iteration (queue.py:87-95), before the row is rewritten
     int32_t popped = VL_MAXINT;
     if constexpr (FUSED) {
-        const int32_t *li = reinterpret_cast<const int32_t *>(uk);
-        const float *ld = reinterpret_cast<const float *>(li + a.m);
-        for (int i = threadIdx.x; i < a.m; i += blockDim.x) raw[i] = vl_make_key(li[i], ld[i]);
         if (threadIdx.x < kWave && (int)threadIdx.x < a.Vt) popped = g_visit_s[threadIdx.x];
         if (threadIdx.x == 0) {
             n_new_s = 0;
@@ -494,6 +502,13 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
         if (threadIdx.x == 0 && n_new) a.seen_count[row] = cnt;
     }
     if (threadIdx.x == 0) raise_running_max(first_next, cnt, min(a.E, a.Vt * t));
+    if constexpr (FUSED) {
+        refine(seen_b, cnt, seen_full, qa[a.L - 1], nva > 0 ? va[nva - 1] : 0ull, fl, red);
+        // a thread packs the slots it (or a lane of its own wavefront, before the barrier above or in refine) wrote
+        const int32_t *li = reinterpret_cast<const int32_t *>(uk);
+        const float *ld = reinterpret_cast<const float *>(li + a.m);
+        for (int i = threadIdx.x; i < a.m; i += blockDim.x) raw[i] = vl_make_key(li[i], ld[i]);
+    }
 
     // ---- which candidates can matter at all -------------------------------------------
     // search queue: only keys below its last slot can enter.  visit queue (VL slots, Vt of
@@ -654,6 +669,9 @@ struct StepArgs {
     int memo_min_rate;    // the cache stays in use only if that share is at least this (x 256)
     int count_evals;
     int l2;  // 0: cosine distance, 1: squared L2
+    const uint8_t *sketch;     // 8-bit sketch of `vectors` (sketch_device.h), or null
+    int64_t sketch_row_bytes;
+    int sketch_chunks;         // 16-byte chunks of data in a sketch row
 };
 
 // A probe of the distance cache is a random 8-byte read and every evaluated distance a random 8-byte
@@ -670,7 +688,12 @@ constexpr int kMemoDecide = 9;
 // their remainder the slow way (read, wait, store) - none of the benchmark shapes has one.
 constexpr int kPreQ = 2, kPreV = 2, kPreS = 4;
 
-template <int CPL, int LPR, int U, bool GENERIC, int THREADS>
+// SCPL > 0: the kernel can look at candidates through the sketch first (SCPL chunks per lane, SLPR lanes
+// per sketch row, SU loads in flight).  A row does so once it has left the distance cache alone (a cache
+// hit is cheaper still, so rows whose candidates repeat keep the cache instead): it gets bounds for all
+// candidates from a quarter of the bytes, then exact distances for the few whose lower bound is not above
+// every threshold that decides what the merge phase keeps.
+template <int CPL, int LPR, int U, bool GENERIC, int THREADS, int SCPL = 0, int SLPR = 64, int SU = 1>
 __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
     extern __shared__ __align__(16) unsigned char smem[];
     const MergeArgs &a = s.m;
@@ -741,6 +764,8 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
     const bool resample = memo_row && t == kMemoDecide;
     if (memo_row && memo_rate < s.memo_min_rate) memo_row = nullptr;
     const bool probing = memo_row != nullptr;
+    bool sketching = false;
+    if constexpr (SCPL > 0) sketching = s.memo ? (t > kMemoDecide && !probing) : true;
     if (tid < a.Vt) g_visit_s[tid] = my_visit;
     if (tid == 0) {
         g_n_ex_s = a.excl ? a.excl_cols : 0;
@@ -794,8 +819,28 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
             if (e == VL_MAXINT) atomicMin(&g_n_ex_s, i);
         }
     }
-    int n_wanted = 0, n_fetched = 0;  // counts of this wavefront
-    for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
+    int n_wanted = 0, n_fetched = 0, n_sketched = 0;  // counts of this wavefront
+    float *le = reinterpret_cast<float *>(raw);                     // upper bounds (raw is filled in the merge phase)
+    if constexpr (SCPL > 0) {
+        if (sketching) {
+            SketchQuery<SCPL> sq;
+            sketch_query_load<SCPL, SLPR>(sq, q_row, s.dim);
+            for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
+                if (c0 != wave * kWave) id = resolve(c0);
+                const int slot = c0 + lane;
+                const bool has = slot < a.m;
+                const bool ok = has && id != VL_MAXINT && id >= 0 && (int64_t)id < s.n_vectors;
+                if (has) {
+                    li[slot] = ok ? id : VL_MAXINT;
+                    if (!ok) ld[slot] = VL_MAXFLOAT;
+                }
+                if (s.count_evals) n_sketched += __popcll(__ballot(ok));
+                wave_sketch<SCPL, SLPR, SU>(sq, s.sketch, s.sketch_row_bytes, s.sketch_chunks, id, ok, ld + c0, le + c0);
+            }
+            n_wanted = n_sketched;
+        }
+    }
+    for (int c0 = wave * kWave; c0 < a.m && !sketching; c0 += THREADS) {
         if (c0 != wave * kWave) id = resolve(c0);
         const int slot = c0 + lane;
         const bool has = slot < a.m;
@@ -822,27 +867,106 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
         const int stripe = (int)((blockIdx.x * (THREADS / kWave) + wave) & (kBeamStripes - 1));
         if (n_wanted) atomicAdd(&c->wanted[stripe], (unsigned long long)n_wanted);
         if (n_fetched) atomicAdd(&c->evals[stripe], (unsigned long long)n_fetched);
+        if (n_sketched) atomicAdd(&c->sketched[stripe], (unsigned long long)n_sketched);
     }
     if (resample && lane == 0) {
         atomicAdd(&probe_asked_s, n_wanted);
         atomicAdd(&probe_hits_s, n_wanted - n_fetched);
     }
     __syncthreads();
-    if (resample && tid == 0)
-        s.memo_rate[row] = probe_asked_s > 0 ? (probe_hits_s * 256) / probe_asked_s : 256;
+    if (resample && tid == 0) {
+        const int rate = probe_asked_s > 0 ? (probe_hits_s * 256) / probe_asked_s : 256;
+        s.memo_rate[row] = rate;
+        if (rate < s.memo_min_rate) atomicAdd(&c->cache_dropped, 1);
+    }
     // ---- merge: ann.py:75-88 ----
-    merge_row<THREADS, true>(a, smem, pre);
+    if constexpr (SCPL > 0) {
+        // A sketched row knows every candidate distance only as lo <= d <= hi (ld holds lo, le holds hi).
+        // What the merge phase keeps of the candidates: keys below the search queue's last slot (ws),
+        // unvisited keys below the visit queue's last live slot (wv), and the Vt smallest distinct
+        // unvisited keys above wv.  Let tv be the Vt-th smallest hi among the distinct unvisited candidates
+        // that are certainly above wv (lo > wv): Vt candidates are then known to be at most tv, so a
+        // candidate with lo > tv is not one of the Vt smallest.  Hence a candidate whose lo is above ws, and
+        // which is visited or has lo above both wv and tv, cannot enter either queue and is dropped; all
+        // others are evaluated exactly, by the same code and in the same order as an unsketched row's.
+        // Comparisons are written so that a NaN bound counts as "evaluate".
+        auto refine = [&](const int32_t *seen_b, int cnt, bool seen_full, uint64_t ws, uint64_t wv, uint8_t *flags,
+                          uint64_t *red) {
+            if (!sketching) return;  // uniform over the workgroup
+            const float ws_d = vl_key_dist(ws);
+            const float wv_d = nva > 0 ? vl_key_dist(wv) : -1.0f;
+            for (int i = tid; i < a.m; i += THREADS) {
+                const int32_t cid = li[i];
+                uint8_t f = 0;
+                if (cid != VL_MAXINT) {
+                    const float lo = ld[i];
+                    bool need = !(lo > ws_d);
+                    if (!seen_full && !sorted_contains(seen_b, cnt, cid)) {
+                        if (!(lo > wv_d)) need = true;
+                        else f |= 2;  // unvisited and certainly above the visit queue's last live slot
+                    }
+                    if (need) f |= 4;
+                }
+                flags[i] = f;
+            }
+            float tv = -1.0f;
+            if (!seen_full) {
+                uint64_t last = 0ull;
+                for (int r = 0; r < a.Vt; ++r) {
+                    uint64_t mine = kPadKey;
+                    for (int i = tid; i < a.m; i += THREADS) {
+                        if (!(flags[i] & 2)) continue;
+                        const uint64_t k = vl_make_key(li[i], le[i]);
+                        if ((r == 0 || k > last) && k < mine) mine = k;
+                    }
+                    const uint64_t mn = block_min_key(mine, red, r);
+                    if (mn == kPadKey) {  // fewer than Vt such candidates: every one of them may be taken
+                        tv = __builtin_inff();
+                        break;
+                    }
+                    last = mn;
+                    tv = vl_key_dist(mn);
+                }
+            }
+            int n_exact = 0;
+            for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
+                const int slot = c0 + lane;
+                const bool has = slot < a.m;
+                const int32_t cid = has ? li[slot] : VL_MAXINT;
+                const uint8_t f = has ? flags[slot] : 0;
+                const bool ok = (f & 4) || ((f & 2) && !(ld[slot] > tv));
+                if (has && cid != VL_MAXINT && !ok) {
+                    li[slot] = VL_MAXINT;
+                    ld[slot] = VL_MAXFLOAT;
+                }
+                if (s.count_evals) n_exact += __popcll(__ballot(ok));
+                wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0, nullptr, 0, false);
+            }
+            if (s.count_evals && lane == 0 && n_exact)
+                atomicAdd(&c->evals[(int)((blockIdx.x * (THREADS / kWave) + wave) & (kBeamStripes - 1))],
+                          (unsigned long long)n_exact);
+            __syncthreads();
+        };
+        merge_row<THREADS, true>(a, smem, pre, refine);
+    } else {
+        merge_row<THREADS, true>(a, smem, pre);
+    }
 }
 
-template <int CPL, int LPR, int U, bool GENERIC>
+template <int CPL, int LPR, int U, bool GENERIC, int SCPL = 0, int SLPR = 64, int SU = 1>
 void launch_step(const StepArgs &s, int threads, size_t smem, hipStream_t st) {
     dim3 grid((unsigned)s.m.n_rows);
+    if constexpr (SCPL > 0) {
+        if (!s.sketch) return launch_step<CPL, LPR, U, GENERIC>(s, threads, smem, st);
+    }
     if (threads == 128) {
-        if (vl_allow_lds(beam_step_kernel<CPL, LPR, U, GENERIC, 128>, smem) != hipSuccess) return;  // seen by the launch check
-        hipLaunchKernelGGL((beam_step_kernel<CPL, LPR, U, GENERIC, 128>), grid, dim3(128), smem, st, s);
+        auto kernel = beam_step_kernel<CPL, LPR, U, GENERIC, 128, SCPL, SLPR, SU>;
+        if (vl_allow_lds(kernel, smem) != hipSuccess) return;  // seen by the launch check
+        hipLaunchKernelGGL(kernel, grid, dim3(128), smem, st, s);
     } else {
-        if (vl_allow_lds(beam_step_kernel<CPL, LPR, U, GENERIC, 256>, smem) != hipSuccess) return;
-        hipLaunchKernelGGL((beam_step_kernel<CPL, LPR, U, GENERIC, 256>), grid, dim3(256), smem, st, s);
+        auto kernel = beam_step_kernel<CPL, LPR, U, GENERIC, 256, SCPL, SLPR, SU>;
+        if (vl_allow_lds(kernel, smem) != hipSuccess) return;
+        hipLaunchKernelGGL(kernel, grid, dim3(256), smem, st, s);
     }
 }
 
@@ -856,22 +980,24 @@ int dist_variant() {
     return v;
 }
 
+// The last three numbers are the sketch's lane shape for rows of that size: a sketch row has a quarter of
+// the chunks, so a quarter of the lanes (or of the chunks per lane) covers it.
 int launch_step_by_dim(const StepArgs &s, bool aligned, int threads, size_t smem, hipStream_t st) {
     const int nchunks = s.nchunks;
     const int variant = dist_variant();
     if (!aligned || nchunks > 512) launch_step<1, 64, 1, true>(s, threads, smem, st);
-    else if (nchunks <= 16) launch_step<1, 16, 8, false>(s, threads, smem, st);
+    else if (nchunks <= 16) launch_step<1, 16, 8, false, 1, 8, 8>(s, threads, smem, st);
     else if (nchunks <= 32 && variant == 1) launch_step<1, 32, 8, false>(s, threads, smem, st);
-    else if (nchunks <= 32) launch_step<2, 16, 4, false>(s, threads, smem, st);
-    else if (nchunks <= 64) launch_step<1, 64, 8, false>(s, threads, smem, st);
-    else if (nchunks <= 96 && variant != 1) launch_step<3, 32, 4, false>(s, threads, smem, st);
-    else if (nchunks <= 128) launch_step<2, 64, 8, false>(s, threads, smem, st);
-    else if (nchunks <= 192) launch_step<3, 64, 4, false>(s, threads, smem, st);
-    else if (nchunks <= 256) launch_step<4, 64, 4, false>(s, threads, smem, st);
-    else if (nchunks <= 320) launch_step<5, 64, 2, false>(s, threads, smem, st);
-    else if (nchunks <= 384) launch_step<6, 64, 2, false>(s, threads, smem, st);
-    else if (nchunks <= 448) launch_step<7, 64, 2, false>(s, threads, smem, st);
-    else launch_step<8, 64, 2, false>(s, threads, smem, st);
+    else if (nchunks <= 32) launch_step<2, 16, 4, false, 1, 8, 8>(s, threads, smem, st);
+    else if (nchunks <= 64) launch_step<1, 64, 8, false, 2, 8, 4>(s, threads, smem, st);
+    else if (nchunks <= 96 && variant != 1) launch_step<3, 32, 4, false, 3, 8, 4>(s, threads, smem, st);
+    else if (nchunks <= 128) launch_step<2, 64, 8, false, 2, 16, 4>(s, threads, smem, st);
+    else if (nchunks <= 192) launch_step<3, 64, 4, false, 3, 16, 4>(s, threads, smem, st);
+    else if (nchunks <= 256) launch_step<4, 64, 4, false, 4, 16, 2>(s, threads, smem, st);
+    else if (nchunks <= 320) launch_step<5, 64, 2, false, 3, 32, 4>(s, threads, smem, st);
+    else if (nchunks <= 384) launch_step<6, 64, 2, false, 3, 32, 4>(s, threads, smem, st);
+    else if (nchunks <= 448) launch_step<7, 64, 2, false, 4, 32, 2>(s, threads, smem, st);
+    else launch_step<8, 64, 2, false, 4, 32, 2>(s, threads, smem, st);
     VL_LAUNCH_CHECK("beam_step_kernel");
     return VL_OK;
 }
@@ -934,7 +1060,7 @@ int beam_layout(const vl_beam_params *p, BeamLayout *l, bool lean = false) {
     if (slots > 65536) slots = 65536;
     while (slots > 1024 && p->n_rows * (int64_t)slots * 8 > (8ll << 30)) slots >>= 1;
     if (memo_env >= 0) slots = memo_env;
-    if (lean) slots = 0;
+    if (lean || (p->flags & VL_BEAM_NO_CACHE)) slots = 0;
     l->memo_slots = slots;
     l->off_memo = o; o = align256(o + p->n_rows * (int64_t)slots * 8);
     l->total = o;
@@ -976,7 +1102,8 @@ __global__ void beam_status_kernel(const BeamCtrl *c, int iterations, int R, int
 // status_out[0] = 1 if the loop ended within them (else 0) and status_out[1] = the iteration count.
 int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *queries, const float *vectors,
                   const int32_t *beams, int32_t *q_ids, float *q_dists, const int32_t *exclude, void *workspace,
-                  int64_t workspace_bytes, int64_t fixed_iterations, int32_t *status_out, void *stream) {
+                  int64_t workspace_bytes, int64_t fixed_iterations, int32_t *status_out, void *stream,
+                  const uint8_t *sketch = nullptr) {
     int rc;
     VL_REQUIRE(queries && vectors && beams && q_ids && q_dists && workspace, "null pointer");
     VL_REQUIRE(((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
@@ -1078,6 +1205,25 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
         int64_t r = (205ll * 256) / (4 * p->dim);
         step.memo_min_rate = rate_env >= 0 ? rate_env : (int)(r > 255 ? 255 : r);
     }
+    // The sketch serves the cosine distance of 16-byte aligned rows in the fused step; other calls ignore it.
+    step.sketch = (sketch && !step.l2 && aligned && use_fused && p->dim <= 2048) ? sketch : nullptr;
+    step.sketch_row_bytes = sketch_row_bytes(p->dim);
+    step.sketch_chunks = (int)sketch_data_chunks(p->dim);
+    if (step.sketch) {
+        // With a sketch the alternative to the cache is no longer the whole row.  Per candidate, in bytes: the
+        // cache costs a 64-byte probe, and row + id + a 64-byte store for every miss; the sketch costs its row
+        // + id, and an exact evaluation for about one candidate in twenty.  The cache stays in use only above the
+        // share of hits at which the two are equal (0.72 for 768 columns).
+        static const int rate_env = [] {
+            const char *e = getenv("VL_BEAM_SKETCH_MIN_RATE");
+            return e ? atoi(e) : -1;
+        }();
+        const double row = 4.0 * p->dim + 76.0, sk = (double)step.sketch_row_bytes + 4.0 + 0.05 * (4.0 * p->dim + 12.0);
+        int r = (int)(256.0 * (1.0 - (sk - 64.0) / row));
+        r = r < 0 ? 0 : (r > 255 ? 255 : r);
+        if (r > step.memo_min_rate) step.memo_min_rate = r;
+        if (rate_env >= 0) step.memo_min_rate = rate_env;
+    }
     step.memo_shift = 32;
     if (step.memo) {
         int lg = 0;
@@ -1118,6 +1264,12 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     // queue changes and the next check ends the loop.  More iterations than that mean the
     // control block was overwritten while the loop ran (a workspace shared by two calls).
     const int64_t t_limit = l.E + l.VL + 2 * (int64_t)R + 2;
+    // The kernel that can read the sketch holds more registers, so fewer rows are resident per compute unit:
+    // it is launched only once rows are known to use it.  Rows decide in iteration kMemoDecide (those that
+    // leave the distance cache alone are counted on the device); the host reads the count at its next
+    // progress check.  Without a cache every row uses the sketch from the start.
+    const uint8_t *sketch_table = step.sketch;
+    int sketch_rows_known = (sketch_table && !step.memo) ? 1 : -1;
     int64_t t = 0;
     for (;;) {
         for (int r = 0; r < R; ++r) {
@@ -1126,6 +1278,7 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
             a.iter = (int)t;
             if (use_fused) {
                 step.m = a;
+                step.sketch = sketch_rows_known > 0 ? sketch_table : nullptr;
                 rc = launch_step_by_dim(step, aligned, merge_threads == 128 ? 128 : 256, smem, st);
                 if (rc < 0) return rc;
                 if (prof) VL_HIP(hipEventRecord(ev[3 * r + 1], st));
@@ -1149,6 +1302,9 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
         }
         int changed = 0;
         VL_HIP(hipMemcpyAsync(&changed, &ctrl->changed[(t / R) & 63], sizeof(int), hipMemcpyDeviceToHost, st));
+        const bool ask_dropped = sketch_table && sketch_rows_known < 0 && t >= kMemoDecide;
+        if (ask_dropped)
+            VL_HIP(hipMemcpyAsync(&sketch_rows_known, &ctrl->cache_dropped, sizeof(int), hipMemcpyDeviceToHost, st));
         VL_HIP(hipStreamSynchronize(st));
         if (prof) {
             for (int r = 0; r < R; ++r) {
@@ -1179,10 +1335,13 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
         VL_HIP(hipMemcpyAsync(ev_counts, ctrl->wanted, sizeof(ev_counts), hipMemcpyDeviceToHost, st));
         VL_HIP(hipStreamSynchronize(st));
         for (int i = 0; i < kBeamStripes; ++i) mine.wanted += (int64_t)ev_counts[i];
+        VL_HIP(hipMemcpyAsync(ev_counts, ctrl->sketched, sizeof(ev_counts), hipMemcpyDeviceToHost, st));
+        VL_HIP(hipStreamSynchronize(st));
+        for (int i = 0; i < kBeamStripes; ++i) mine.sketched += (int64_t)ev_counts[i];
         std::lock_guard<std::mutex> hold(g_prof_mutex);
         g_prof.expand_ms += mine.expand_ms; g_prof.merge_ms += mine.merge_ms;
         g_prof.expand_launches += mine.expand_launches; g_prof.merge_launches += mine.merge_launches;
-        g_prof.evals += mine.evals; g_prof.wanted += mine.wanted;
+        g_prof.evals += mine.evals; g_prof.wanted += mine.wanted; g_prof.sketched += mine.sketched;
         g_prof.rows += p->n_rows;
         g_prof.iterations += t;
     }
@@ -1201,6 +1360,19 @@ VL_EXPORT int64_t vl_closest_vectors(const vl_beam_params *p, const float *queri
     if (p->n_rows == 0) return 0;
     return beam_loop(p, l, queries, vectors, beams, q_ids, q_dists, exclude, workspace, workspace_bytes, 0, nullptr,
                      stream);
+}
+
+VL_EXPORT int64_t vl_closest_vectors_with_sketch(const vl_beam_params *p, const float *queries, const float *vectors,
+                                                 const uint8_t *sketch, const int32_t *beams, int32_t *q_ids,
+                                                 float *q_dists, const int32_t *exclude, void *workspace,
+                                                 int64_t workspace_bytes, void *stream) {
+    BeamLayout l;
+    int rc = beam_layout(p, &l);
+    if (rc < 0) return rc;
+    VL_REQUIRE(!sketch || ((uintptr_t)sketch & 15) == 0, "the sketch table must be 16-byte aligned");
+    if (p->n_rows == 0) return 0;
+    return beam_loop(p, l, queries, vectors, beams, q_ids, q_dists, exclude, workspace, workspace_bytes, 0, nullptr,
+                     stream, sketch);
 }
 
 // ---- the entry point that allocates nothing -------------------------------------------
@@ -1266,7 +1438,8 @@ VL_EXPORT int vl_closest_vectors_noalloc(const vl_beam_params *p, const float *q
 // candidate rows are counted.  out[0..7] = expand ms, merge ms, expand
 // launches, merge launches, candidate rows fetched, query rows, iterations,
 // candidate distances asked for (fetched + served by the per-row cache),
-// summed since the last reset.
+// out[8] = candidate rows looked at through the sketch, summed since the last
+// reset.
 VL_EXPORT int vl_beam_profile(int enable, int reset, double *out) {
     std::lock_guard<std::mutex> hold(g_prof_mutex);
     if (out) {
@@ -1274,6 +1447,7 @@ VL_EXPORT int vl_beam_profile(int enable, int reset, double *out) {
         out[2] = (double)g_prof.expand_launches; out[3] = (double)g_prof.merge_launches;
         out[4] = (double)g_prof.evals; out[5] = (double)g_prof.rows; out[6] = (double)g_prof.iterations;
         out[7] = (double)g_prof.wanted;
+        out[8] = (double)g_prof.sketched;
     }
     if (reset) g_prof = BeamProfile();
     g_prof.enabled = enable;

@@ -1,0 +1,96 @@
+// Builds the 8-bit sketch of a vector table (layout and use: sketch_device.h).  No counterpart in the
+// reference, which evaluates every candidate distance in full (kernels.py:204-257).
+#include "sketch_device.h"
+
+namespace {
+
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+    for (int h = kWave / 2; h >= 1; h >>= 1) x = fmaxf(x, __shfl_xor(x, h));
+    return x;
+}
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int h = kWave / 2; h >= 1; h >>= 1) x += __shfl_xor(x, h);
+    return x;
+}
+
+// One wavefront per row; a lane packs four elements into one 32-bit store.
+__global__ __launch_bounds__(256) void sketch_build_kernel(const float *__restrict__ vectors, int64_t n, int dim,
+                                                           int64_t row0, uint8_t *__restrict__ table) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t row = row0 + (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+    if (row >= n) return;
+    const float *v = vectors + row * dim;
+    const int chunks = (int)sketch_data_chunks(dim);
+    uint8_t *out = table + row * sketch_row_bytes(dim);
+
+    float mx = 0.f;
+    bool finite = true;
+    for (int j = lane; j < dim; j += kWave) {
+        const float x = v[j];
+        finite = finite && (x - x == 0.0f);  // false for NaN and for either infinity
+        mx = fmaxf(mx, __builtin_fabsf(x));
+    }
+    mx = wave_max(mx);
+    finite = __ballot(!finite) == 0;
+    const float scale = mx / 127.0f;
+    const float inv = mx > 0.f ? 127.0f / mx : 0.f;
+
+    float r2 = 0.f, n2 = 0.f;
+    for (int g = lane; g < chunks * 4; g += kWave) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int j = 4 * g + k;
+            float qv = 0.f;
+            if (j < dim) {
+                const float x = v[j];
+                qv = fminf(fmaxf(rintf(x * inv), -127.0f), 127.0f);
+                const float e = x - scale * qv;
+                r2 = __builtin_fmaf(e, e, r2);
+                n2 = __builtin_fmaf(x, x, n2);
+            }
+            word |= (uint32_t)((int)qv + 128) << (8 * k);
+        }
+        reinterpret_cast<uint32_t *>(out)[g] = word;
+    }
+    r2 = wave_sum(r2);
+    n2 = wave_sum(n2);
+    if (lane == 0) {
+        // 1.001: the float32 sums above are off by at most dim * 2^-24 of their value, the products
+        // scale * q by 2^-24 of |v_j|; the floor covers squares that underflow (elements below 1e-19);
+        // a row that holds a NaN or an infinity promises nothing
+        const float floor_ = 1.1e-19f * __builtin_sqrtf((float)dim);
+        float4 tail;
+        tail.x = finite ? scale : 0.f;
+        tail.y = finite ? __builtin_sqrtf(r2) * 1.001f + floor_ : __builtin_inff();
+        tail.z = finite ? __builtin_sqrtf(n2) * 1.001f + floor_ : __builtin_inff();
+        tail.w = 0.f;
+        *reinterpret_cast<float4 *>(out + (int64_t)chunks * 16) = tail;
+    }
+}
+
+}  // namespace
+
+VL_EXPORT int64_t vl_sketch_row_bytes(int64_t dim) {
+    if (dim <= 0) {
+        vl_set_error("dim must be positive");
+        return VL_ERR_ARG;
+    }
+    return sketch_row_bytes(dim);
+}
+
+VL_EXPORT int vl_sketch_build(const float *vectors, int64_t n_vectors, int64_t dim, uint8_t *table, void *stream) {
+    VL_REQUIRE(vectors && table, "null pointer");
+    VL_REQUIRE(n_vectors >= 0 && dim > 0 && dim < (1 << 24), "bad sizes");
+    VL_REQUIRE(((uintptr_t)table & 15) == 0, "the sketch table must be 16-byte aligned");
+    const int rows_per_block = 256 / kWave;
+    for (int64_t row0 = 0; row0 < n_vectors; row0 += kMaxBlocks * rows_per_block) {
+        int64_t rows = n_vectors - row0 < kMaxBlocks * rows_per_block ? n_vectors - row0 : kMaxBlocks * rows_per_block;
+        hipLaunchKernelGGL(sketch_build_kernel, dim3((unsigned)((rows + rows_per_block - 1) / rows_per_block)), dim3(256),
+                           0, (hipStream_t)stream, vectors, n_vectors, (int)dim, row0, table);
+        VL_LAUNCH_CHECK("sketch_build_kernel");
+    }
+    return VL_OK;
+}

@@ -54,6 +54,10 @@ _SIGNATURES = {
     "vl_beam_workspace_bytes": (C.c_int64, [C.POINTER(BeamParams)]),
     "vl_closest_vectors": (C.c_int64, [C.POINTER(BeamParams), _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr]),
     "vl_closest_vectors_noalloc": (C.c_int, [C.POINTER(BeamParams), _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr]),
+    "vl_closest_vectors_with_sketch": (C.c_int64, [C.POINTER(BeamParams), _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
+                                                   _i64, _ptr]),
+    "vl_sketch_row_bytes": (C.c_int64, [_i64]),
+    "vl_sketch_build": (C.c_int, [_ptr, _i64, _i64, _ptr, _ptr]),
     "vl_beam_profile": (C.c_int, [C.c_int, C.c_int, C.POINTER(C.c_double)]),
     "vl_optimize_graph_workspace_bytes": (C.c_int64, [_i64, _i64, _i64]),
     "vl_optimize_graph": (C.c_int, [_ptr, _i64, _i64, _i64, _ptr, _ptr, _i64, _ptr]),

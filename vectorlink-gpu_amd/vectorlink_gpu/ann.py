@@ -15,7 +15,8 @@ from torch import Tensor
 
 from . import _native as nv
 from .constants import DEVICE, MAXFLOAT, MAXINT
-from .kernels import calculate_distances, gather_distances, knn_exact, optimize_graph, prune_, search_from_seeds
+from .kernels import (build_sketch, calculate_distances, gather_distances, knn_exact, optimize_graph, prune_,
+                      search_from_seeds, sketch_row_bytes)
 from . import log as _log
 from .log import log_time
 from .queue import Queue
@@ -25,6 +26,7 @@ from .utils import add_new_to_seen_, generate_circulant_beams, generate_queue_ci
 BEAM_TWO_LAUNCHES = 1  # include/vlgpu.h: VL_BEAM_TWO_LAUNCHES
 BEAM_SORT_MERGE = 2    # include/vlgpu.h: VL_BEAM_SORT_MERGE
 BEAM_PER_QUERY_STOP = 4  # include/vlgpu.h: VL_BEAM_PER_QUERY_STOP (a different loop: every row stops on its own)
+BEAM_NO_CACHE = 8  # include/vlgpu.h: VL_BEAM_NO_CACHE (no per-row cache of evaluated distances; same result)
 
 
 def _beam_params(batch: int, dim: int, n_vectors: int, width: int, queue: Queue, config: Dict,
@@ -131,7 +133,7 @@ def closest_vectors_stepwise(query_vecs: Tensor, search_queue: Queue, vectors: T
 
 @log_time
 def closest_vectors(query_vecs: Tensor, search_queue: Queue, vectors: Tensor, beams: Tensor, config: Dict,
-                    exclude: Optional[Tensor] = None, flags: int = 0) -> int:
+                    exclude: Optional[Tensor] = None, flags: int = 0, sketch: Optional[Tensor] = None) -> int:
     """reference ann.py:38-93.  Updates search_queue in place; returns the
     number of iterations run (the reference returns True).  Rows are exact on
     [:, :search_queue.length]; the slots beyond are unspecified.  flags picks
@@ -143,7 +145,12 @@ def closest_vectors(query_vecs: Tensor, search_queue: Queue, vectors: Tensor, be
     (distance, id) with distinct ids, and an id carrying the same distance
     wherever it occurs, i.e. the queue's distances are distances to `vectors`
     rows under this call's query rows.  For a queue in any other state pass
-    BEAM_SORT_MERGE, which sorts whole rows like the reference does."""
+    BEAM_SORT_MERGE, which sorts whole rows like the reference does.
+
+    sketch (an addition): the 8-bit sketch of `vectors` from kernels.build_sketch.
+    Rows whose candidates rarely repeat then look at their candidates through the
+    sketch first and fetch only the rows that can still enter a queue; the
+    result is the same, bit for bit."""
     assert query_vecs.dtype == torch.float32 and vectors.dtype == torch.float32 and beams.dtype == torch.int32
     nv.require_gpu(query_vecs, vectors, beams, search_queue.indices, exclude)
     query_vecs = query_vecs.contiguous()
@@ -161,9 +168,13 @@ def closest_vectors(query_vecs: Tensor, search_queue: Queue, vectors: Tensor, be
     workspace = _workspace(vectors.device)
     with workspace.lock:
         ws = workspace.reserve(need, vectors.device)
-        iterations = nv.check(nv.lib().vl_closest_vectors(
-            ctypes.byref(p), nv.ptr(query_vecs), nv.ptr(vectors), nv.ptr(beams), nv.ptr(search_queue.indices),
-            nv.ptr(search_queue.distances), nv.ptr(excl), nv.ptr(ws), ws.numel(), nv.stream()))
+        if sketch is not None:
+            assert sketch.dtype == torch.uint8 and sketch.is_contiguous() and sketch.is_cuda
+            assert sketch.size() == (vectors.size(0), sketch_row_bytes(dim)), "not a sketch of these vectors"
+        iterations = nv.check(nv.lib().vl_closest_vectors_with_sketch(
+            ctypes.byref(p), nv.ptr(query_vecs), nv.ptr(vectors), nv.ptr(sketch), nv.ptr(beams),
+            nv.ptr(search_queue.indices), nv.ptr(search_queue.distances), nv.ptr(excl), nv.ptr(ws), ws.numel(),
+            nv.stream()))
     with _WORKSPACES_LOCK:
         _log.BEAM_ITERATIONS += iterations
     return iterations
@@ -210,6 +221,12 @@ class GraphBuild:
             (self.beams, self.beam_distances) = initial
             assert self.beams.size() == (self.num_vecs, self.queue_length) == self.beam_distances.size()
         self.distances = self.beam_distances
+        # 8-bit sketch of the vectors (an addition; config["sketch"] = False turns it off): the first loop's
+        # searches sample the table almost at random and keep few of their candidates, which the sketch
+        # finds out for a quarter of the traffic.  The graph does not depend on it.
+        self.sketch = None
+        if config.get("sketch", True) and not stale_distances and config.get("metric", "cosine") == "cosine":
+            self.sketch = build_sketch(vectors)
         self.stats: list = []  # one dict per finished optimisation loop
         self.history: Optional[list] = [] if keep_history else None
         self.finished = False
@@ -240,7 +257,10 @@ class GraphBuild:
                     exclude = excluding_self(start, end, ql, device)
                     queue = Queue(end - start, ql, ql + remaining_capacity, device=device)
                     queue.insert(self.beams.narrow(0, start, end - start), seed_distances.narrow(0, start, end - start))
-                    t = search(vectors[start:end], queue, vectors, self.beams, config, exclude)
+                    if self.sketch is not None:
+                        t = search(vectors[start:end], queue, vectors, self.beams, config, exclude, sketch=self.sketch)
+                    else:
+                        t = search(vectors[start:end], queue, vectors, self.beams, config, exclude)
                     next_beams.narrow(0, start, end - start).copy_(queue.indices.narrow(1, 0, ql))
                     next_beam_distances.narrow(0, start, end - start).copy_(queue.distances.narrow(1, 0, ql))
                     stream.synchronize()

@@ -178,6 +178,25 @@ def knn_exact(queries: Tensor, vectors: Tensor, k: int, metric: str = "cosine") 
     return (ids, dists)
 
 
+def sketch_row_bytes(dim: int) -> int:
+    """Bytes of one row of the 8-bit sketch of [N, dim] vectors."""
+    return nv.check(nv.lib().vl_sketch_row_bytes(dim))
+
+
+def build_sketch(vectors: Tensor) -> Tensor:
+    """8-bit sketch of `vectors` (no counterpart in the reference): per row the
+    elements rounded to 8 bits with one scale, and how far the rounding moved the
+    row, which bounds every dot product with it.  [N, sketch_row_bytes(dim)] uint8;
+    closest_vectors(..., sketch=...) uses it to decide which candidate rows to
+    fetch; no distance it returns comes from the sketch."""
+    _check_f32(vectors, "vectors")
+    nv.require_gpu(vectors)
+    (n, dim) = vectors.size()
+    out = torch.empty((n, sketch_row_bytes(dim)), dtype=torch.uint8, device=vectors.device)
+    nv.check(nv.lib().vl_sketch_build(nv.ptr(vectors), n, dim, nv.ptr(out), nv.stream()))
+    return out
+
+
 def optimize_graph(beams: Tensor, degree: int) -> Tensor:
     """Rank-based graph optimisation (not in the reference): re-order every row of
     `beams` ([N, W], best first, MAXINT = empty) by the number of two-hop detours
