@@ -65,18 +65,23 @@ def profile_read(nv, reset=True, enable=1):
 
 def step_roofline(prof, dim, batch_rows):
     """Algorithmic bytes of the beam-search step from the hook counters: 4*dim + 12 per candidate row actually
-    fetched and evaluated, plus the query row (4*dim) once per (row, iteration)."""
+    fetched and evaluated, a sketch row + the id (16*ceil(dim/16) + 16 + 4) per candidate looked at through the
+    8-bit sketch, plus the query row (4*dim) once per (row, iteration)."""
     launches = max(prof["expand_launches"], 1.0)
     per_eval = 4 * dim + 12
+    per_sketch = 16 * ((dim + 15) // 16) + 16 + 4
     q_loads = prof["iterations"] * batch_rows * 4.0 * dim
-    algo = prof["evals"] * per_eval + q_loads
+    algo = prof["evals"] * per_eval + prof["sketched"] * per_sketch + q_loads
     secs = prof["expand_ms"] / 1e3
     gbs = algo / secs / 1e9 if secs > 0 else 0.0
     ref_equiv = (prof["wanted"] * per_eval + q_loads) / secs / 1e9 if secs > 0 else 0.0
+    wanted = max(prof["wanted"], 1.0)
     return dict(launches=int(prof["expand_launches"]), avg_launch_ms=prof["expand_ms"] / launches,
                 algorithmic_bytes_per_launch=algo / launches, achieved_gbs=gbs, frac=gbs / HBM_PEAK_GBS,
                 reference_equivalent_gbs=ref_equiv,
-                distances_served_from_cache=1.0 - prof["evals"] / max(prof["wanted"], 1.0))
+                candidate_rows_fetched=prof["evals"] / wanted,
+                candidates_through_the_sketch=prof["sketched"] / wanted,
+                distances_served_from_cache=(1.0 - prof["evals"] / wanted) if prof["sketched"] == 0 else None)
 
 
 def measured_read_gbs(torch, dev):
@@ -355,7 +360,8 @@ def main():
     per_loop = []
     for li, tables in enumerate(build.history):
         profile_read(nv, reset=True, enable=1)
-        rb = GraphBuild(vectors, cfg, initial=tables, concurrent_batches=1)  # one launch at a time under the events
+        # one launch at a time under the events; the first loop starts from the circulant graph, as in the build
+        rb = GraphBuild(vectors, cfg, initial=tables if li > 0 else None, concurrent_batches=1)
         for i, _ in enumerate(rb.steps()):
             if i + 1 >= replay:
                 break

@@ -667,6 +667,7 @@ struct StepArgs {
     int memo_shift;
     int32_t *memo_rate;   // per row: share (x 256) of the candidates of iteration kMemoDecide that were cached
     int memo_min_rate;    // the cache stays in use only if that share is at least this (x 256)
+    int sketch_min_rate;  // rows whose share is below this (x 256) are counted in the control block (0: nobody counts)
     int count_evals;
     int l2;  // 0: cosine distance, 1: squared L2
     const uint8_t *sketch;     // 8-bit sketch of `vectors` (sketch_device.h), or null
@@ -877,7 +878,7 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
     if (resample && tid == 0) {
         const int rate = probe_asked_s > 0 ? (probe_hits_s * 256) / probe_asked_s : 256;
         s.memo_rate[row] = rate;
-        if (rate < s.memo_min_rate) atomicAdd(&c->cache_dropped, 1);
+        if (rate < s.sketch_min_rate) atomicAdd(&c->cache_dropped, 1);
     }
     // ---- merge: ann.py:75-88 ----
     if constexpr (SCPL > 0) {
@@ -1209,21 +1210,23 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     step.sketch = (sketch && !step.l2 && aligned && use_fused && p->dim <= 2048) ? sketch : nullptr;
     step.sketch_row_bytes = sketch_row_bytes(p->dim);
     step.sketch_chunks = (int)sketch_data_chunks(p->dim);
+    // With a sketch the alternative to the cache is no longer the whole row.  Per candidate, in bytes: the cache
+    // costs a 64-byte probe, and row + id + a 64-byte store for every miss; the sketch costs its row + id, and an
+    // exact evaluation for about one candidate in ten.  Above the share of hits at which the two are equal (0.66
+    // for 768 columns) a row is better off with the cache.
+    int sketch_rate = 0;
     if (step.sketch) {
-        // With a sketch the alternative to the cache is no longer the whole row.  Per candidate, in bytes: the
-        // cache costs a 64-byte probe, and row + id + a 64-byte store for every miss; the sketch costs its row
-        // + id, and an exact evaluation for about one candidate in twenty.  The cache stays in use only above the
-        // share of hits at which the two are equal (0.72 for 768 columns).
         static const int rate_env = [] {
             const char *e = getenv("VL_BEAM_SKETCH_MIN_RATE");
             return e ? atoi(e) : -1;
         }();
-        const double row = 4.0 * p->dim + 76.0, sk = (double)step.sketch_row_bytes + 4.0 + 0.05 * (4.0 * p->dim + 12.0);
+        const double row = 4.0 * p->dim + 76.0, sk = (double)step.sketch_row_bytes + 4.0 + 0.10 * (4.0 * p->dim + 12.0);
         int r = (int)(256.0 * (1.0 - (sk - 64.0) / row));
         r = r < 0 ? 0 : (r > 255 ? 255 : r);
-        if (r > step.memo_min_rate) step.memo_min_rate = r;
-        if (rate_env >= 0) step.memo_min_rate = rate_env;
+        sketch_rate = r > step.memo_min_rate ? r : step.memo_min_rate;
+        if (rate_env >= 0) sketch_rate = rate_env;
     }
+    step.sketch_min_rate = sketch_rate;
     step.memo_shift = 32;
     if (step.memo) {
         int lg = 0;
@@ -1264,10 +1267,13 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     // queue changes and the next check ends the loop.  More iterations than that mean the
     // control block was overwritten while the loop ran (a workspace shared by two calls).
     const int64_t t_limit = l.E + l.VL + 2 * (int64_t)R + 2;
-    // The kernel that can read the sketch holds more registers, so fewer rows are resident per compute unit:
-    // it is launched only once rows are known to use it.  Rows decide in iteration kMemoDecide (those that
-    // leave the distance cache alone are counted on the device); the host reads the count at its next
-    // progress check.  Without a cache every row uses the sketch from the start.
+    // The kernel that can read the sketch holds more registers, so fewer rows are resident per compute unit, and
+    // one launch serves the whole batch: it takes over only when most rows of the batch are better off with the
+    // sketch than with the cache.  Rows measure their share of cache hits in iteration kMemoDecide and those
+    // below the sketch's break-even share are counted on the device; the host reads the count at its next
+    // progress check.  If they are the majority, the break-even share of the sketch becomes the one that rows
+    // apply (rows below it leave the cache alone and use the sketch, the others keep the cache); otherwise the
+    // batch goes on as it would without a sketch.  Without a cache every row uses the sketch from the start.
     const uint8_t *sketch_table = step.sketch;
     int sketch_rows_known = (sketch_table && !step.memo) ? 1 : -1;
     int64_t t = 0;
@@ -1306,6 +1312,10 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
         if (ask_dropped)
             VL_HIP(hipMemcpyAsync(&sketch_rows_known, &ctrl->cache_dropped, sizeof(int), hipMemcpyDeviceToHost, st));
         VL_HIP(hipStreamSynchronize(st));
+        if (ask_dropped) {
+            if (2 * (int64_t)sketch_rows_known >= p->n_rows) step.memo_min_rate = step.sketch_min_rate;
+            else sketch_rows_known = 0;
+        }
         if (prof) {
             for (int r = 0; r < R; ++r) {
                 float ms = 0;

@@ -213,6 +213,7 @@ class GraphBuild:
         device = vectors.device
         self.beam_size = config["beam_size"]
         self.queue_length = self.beam_size * config["beam_queue_factor"]
+        self.circulant_start = initial is None
         if initial is None:
             neighbor_primes = primes(self.queue_length, device)
             self.beams = generate_circulant_beams(self.num_vecs, neighbor_primes)
@@ -258,7 +259,11 @@ class GraphBuild:
                     queue = Queue(end - start, ql, ql + remaining_capacity, device=device)
                     queue.insert(self.beams.narrow(0, start, end - start), seed_distances.narrow(0, start, end - start))
                     if self.sketch is not None:
-                        t = search(vectors[start:end], queue, vectors, self.beams, config, exclude, sketch=self.sketch)
+                        # the neighbour lists of a circulant graph share nothing, so a search of it meets hardly
+                        # any candidate twice: no distance cache, the sketch from the first iteration
+                        first = BEAM_NO_CACHE if (loop == 0 and self.circulant_start) else 0
+                        t = search(vectors[start:end], queue, vectors, self.beams, config, exclude, flags=first,
+                                   sketch=self.sketch)
                     else:
                         t = search(vectors[start:end], queue, vectors, self.beams, config, exclude)
                     next_beams.narrow(0, start, end - start).copy_(queue.indices.narrow(1, 0, ql))
