@@ -108,16 +108,19 @@ __global__ void beam_memo_clear_kernel(uint64_t *memo, int64_t n) {
         memo[i] = (uint64_t)(uint32_t)VL_MAXINT;
 }
 
+// row_word: what every row starts with in its word of the memo_rate array (StepArgs); sketch_rows: how many rows
+// that makes users of the sketch.
 __global__ __launch_bounds__(kQueueThreads) void beam_init_kernel(BeamCtrl *ctrl, int64_t n_rows, const int32_t *q_ids,
                                                                  const float *q_d, int cap, int head, int32_t *v_ids,
                                                                  float *v_d, int VL, int32_t *seen_count,
-                                                                 int32_t *row_quiet) {
+                                                                 int32_t *row_quiet, int32_t *memo_rate, int row_word,
+                                                                 int sketch_rows) {
     int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t == 0) {
         ctrl->stop = 0;
         ctrl->ended_after = 0;
         ctrl->first[0] = ctrl->first[1] = ctrl->first[2] = 0;
-        ctrl->cache_dropped = 0;
+        ctrl->sketch_rows = sketch_rows;
     }
     if (t < 64) ctrl->changed[t] = 0;
     if (t < kBeamStripes) {
@@ -128,6 +131,7 @@ __global__ __launch_bounds__(kQueueThreads) void beam_init_kernel(BeamCtrl *ctrl
     if (t < n_rows) {
         seen_count[t] = 0;
         row_quiet[t] = 0;
+        memo_rate[t] = row_word;
     }
     if (t < n_rows * VL) {  // Queue.initialize_from_queue, queue.py:30-35
         int64_t r = t / VL;
@@ -380,9 +384,14 @@ struct NoRefine {
     __device__ __forceinline__ void operator()(const int32_t *, int, bool, uint64_t, uint64_t, uint8_t *, uint64_t *) const {}
 };
 
-template <int THREADS, bool FUSED, class Refine = NoRefine>
+// kept (fused step only): told how many candidates of the row the merge phase keeps for its queues.
+struct NoCount {
+    __device__ __forceinline__ void operator()(int) const {}
+};
+
+template <int THREADS, bool FUSED, class Refine = NoRefine, class Kept = NoCount>
 __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *smem, RowState pre = RowState{0, 0},
-                                          Refine refine = Refine()) {
+                                          Refine refine = Refine(), Kept kept = Kept()) {
     const int Pc = a.Pc;
     uint64_t *raw = reinterpret_cast<uint64_t *>(smem);  // candidate keys as they arrive
     uint64_t *uk = raw + Pc;                             // the candidates that can matter, then sorted
@@ -553,6 +562,7 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
         return (f & 1) || ((f & 2) && raw[i] <= sel_max);
     };
     const int n_u = block_compact(raw, a.m, uk, wanted, wave_cnt);
+    kept(n_u);
     int Pu = 2;
     while (Pu < n_u) Pu <<= 1;
     for (int i = n_u + threadIdx.x; i < Pu; i += blockDim.x) uk[i] = kPadKey;
@@ -665,7 +675,7 @@ struct StepArgs {
     uint32_t width_magic;  // floor(2^32 / width) + 1: slot / width == umulhi(slot, width_magic) for slot * width < 2^32
     uint64_t *memo;
     int memo_shift;
-    int32_t *memo_rate;   // per row: share (x 256) of the candidates of iteration kMemoDecide that were cached
+    int32_t *memo_rate;   // per row: share (x 256) of the candidates of iteration kMemoDecide that were cached; bit 16: the row prefers the sketch
     int memo_min_rate;    // the cache stays in use only if that share is at least this (x 256)
     int sketch_min_rate;  // rows whose share is below this (x 256) are counted in the control block (0: nobody counts)
     int count_evals;
@@ -718,7 +728,8 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
     pre.cnt = a.seen_count[row];
     pre.first = c->first[t % 3];
     const int quiet = a.row_quiet ? a.row_quiet[row] : 0;
-    const int memo_rate = (s.memo && t > kMemoDecide) ? s.memo_rate[row] : 256;
+    const int memo_word = s.memo_rate[row];
+    const int memo_rate = memo_word & 0xffff;
     int32_t pq_i[kPreQ], pv_i[kPreV], ps[kPreS];
     float pq_d[kPreQ], pv_d[kPreV];
 #pragma unroll
@@ -764,9 +775,10 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
     __shared__ int probe_hits_s, probe_asked_s;
     const bool resample = memo_row && t == kMemoDecide;
     if (memo_row && memo_rate < s.memo_min_rate) memo_row = nullptr;
-    const bool probing = memo_row != nullptr;
     bool sketching = false;
-    if constexpr (SCPL > 0) sketching = s.memo ? (t > kMemoDecide && !probing) : true;
+    if constexpr (SCPL > 0) sketching = (memo_word >> 16) != 0;
+    if (sketching) memo_row = nullptr;
+    const bool probing = memo_row != nullptr;
     if (tid < a.Vt) g_visit_s[tid] = my_visit;
     if (tid == 0) {
         g_n_ex_s = a.excl ? a.excl_cols : 0;
@@ -875,11 +887,21 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
         atomicAdd(&probe_hits_s, n_wanted - n_fetched);
     }
     __syncthreads();
-    if (resample && tid == 0) {
-        const int rate = probe_asked_s > 0 ? (probe_hits_s * 256) / probe_asked_s : 256;
-        s.memo_rate[row] = rate;
-        if (rate < s.sketch_min_rate) atomicAdd(&c->cache_dropped, 1);
+    int measured_rate = 256;
+    if (resample) {
+        measured_rate = probe_asked_s > 0 ? (probe_hits_s * 256) / probe_asked_s : 256;
+        if (tid == 0) s.memo_rate[row] = measured_rate;
     }
+    // A row would rather use the sketch than the cache when few of its candidates repeat (its share of cache
+    // hits is below the sketch's break-even share) AND few of them matter: the merge phase keeps the candidates
+    // below the queues' last slots, which are the ones a sketched row has to evaluate exactly anyway - if that
+    // is more than a quarter of them (a row searching real neighbour lists), the sketch saves nothing.
+    auto kept = [&](int n_kept) {
+        if (resample && tid == 0 && measured_rate < s.sketch_min_rate && 4 * n_kept < a.m) {
+            s.memo_rate[row] = measured_rate | (1 << 16);
+            atomicAdd(&c->sketch_rows, 1);
+        }
+    };
     // ---- merge: ann.py:75-88 ----
     if constexpr (SCPL > 0) {
         // A sketched row knows every candidate distance only as lo <= d <= hi (ld holds lo, le holds hi).
@@ -929,7 +951,7 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
                     tv = vl_key_dist(mn);
                 }
             }
-            int n_exact = 0;
+            int n_exact = 0, n_real = 0;
             for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
                 const int slot = c0 + lane;
                 const bool has = slot < a.m;
@@ -940,17 +962,34 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
                     li[slot] = VL_MAXINT;
                     ld[slot] = VL_MAXFLOAT;
                 }
-                if (s.count_evals) n_exact += __popcll(__ballot(ok));
+                n_exact += __popcll(__ballot(ok));
+                n_real += __popcll(__ballot(cid != VL_MAXINT));
                 wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0, nullptr, 0, false);
             }
             if (s.count_evals && lane == 0 && n_exact)
                 atomicAdd(&c->evals[(int)((blockIdx.x * (THREADS / kWave) + wave) & (kBeamStripes - 1))],
                           (unsigned long long)n_exact);
-            __syncthreads();
+            // A row that has to evaluate more than half of its candidates exactly after all (its candidates lie
+            // within the sketch's error of the queues' last slots: real neighbour lists) gives the sketch up for
+            // the rest of the call.  Not before iteration kMemoDecide: the first iterations fill the visit queue
+            // and keep everything.
+            if (t > kMemoDecide) {
+                if (lane == 0) {
+                    atomicAdd(&probe_asked_s, n_real);
+                    atomicAdd(&probe_hits_s, n_exact);
+                }
+                __syncthreads();
+                if (tid == 0 && 2 * probe_hits_s > probe_asked_s) {
+                    s.memo_rate[row] = memo_rate;
+                    atomicAdd(&c->sketch_rows, -1);
+                }
+            } else {
+                __syncthreads();
+            }
         };
-        merge_row<THREADS, true>(a, smem, pre, refine);
+        merge_row<THREADS, true>(a, smem, pre, refine, kept);
     } else {
-        merge_row<THREADS, true>(a, smem, pre);
+        merge_row<THREADS, true>(a, smem, pre, NoRefine(), kept);
     }
 }
 
@@ -1127,21 +1166,7 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     int32_t *row_quiet = (int32_t *)(ws + l.off_row_quiet);
     BeamCtrl *ctrl = (BeamCtrl *)(ws + l.off_ctrl);
 
-    {
-        int64_t n = p->n_rows * l.VL;
-        if (n < kBeamStripes) n = kBeamStripes;
-        if (n < p->n_rows) n = p->n_rows;
-        hipLaunchKernelGGL(beam_init_kernel, dim3((unsigned)((n + kQueueThreads - 1) / kQueueThreads)),
-                           dim3(kQueueThreads), 0, st, ctrl, p->n_rows, q_ids, q_dists, (int)p->queue_capacity,
-                           (int)l.head, v_ids, v_d, (int)l.VL, seen_count, row_quiet);
-        VL_LAUNCH_CHECK("beam_init_kernel");
-    }
     uint64_t *memo = (uint64_t *)(ws + l.off_memo);
-    if (l.memo_slots > 0) {
-        hipLaunchKernelGGL(beam_memo_clear_kernel, dim3(4096), dim3(256), 0, st, memo, p->n_rows * (int64_t)l.memo_slots);
-        VL_LAUNCH_CHECK("beam_memo_clear_kernel");
-    }
-
     MergeArgs a;
     a.ctrl = ctrl; a.readahead = (int)p->speculative_readahead; a.n_rows = p->n_rows;
     a.cand_ids = cand_ids; a.cand_d = cand_d; a.m = (int)l.m;
@@ -1234,6 +1259,23 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
         VL_REQUIRE((1 << lg) == l.memo_slots, "memo slots must be a power of two");
         step.memo_shift = 32 - lg;
     }
+    // every row starts with the sketch when there is one and no cache to prefer
+    const bool sketch_from_start = step.sketch && !step.memo;
+    {
+        int64_t n = p->n_rows * l.VL;
+        if (n < kBeamStripes) n = kBeamStripes;
+        if (n < p->n_rows) n = p->n_rows;
+        hipLaunchKernelGGL(beam_init_kernel, dim3((unsigned)((n + kQueueThreads - 1) / kQueueThreads)),
+                           dim3(kQueueThreads), 0, st, ctrl, p->n_rows, q_ids, q_dists, (int)p->queue_capacity,
+                           (int)l.head, v_ids, v_d, (int)l.VL, seen_count, row_quiet, (int32_t *)(ws + l.off_memo_rate),
+                           sketch_from_start ? (256 | (1 << 16)) : 256, sketch_from_start ? (int)p->n_rows : 0);
+        VL_LAUNCH_CHECK("beam_init_kernel");
+    }
+    if (l.memo_slots > 0) {
+        hipLaunchKernelGGL(beam_memo_clear_kernel, dim3(4096), dim3(256), 0, st, memo, p->n_rows * (int64_t)l.memo_slots);
+        VL_LAUNCH_CHECK("beam_memo_clear_kernel");
+    }
+
     const int R = (int)p->speculative_readahead;
     if (fixed_iterations > 0) {
         VL_REQUIRE(use_fused, "a fixed number of iterations is only built for the fused step");
@@ -1268,14 +1310,12 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     // control block was overwritten while the loop ran (a workspace shared by two calls).
     const int64_t t_limit = l.E + l.VL + 2 * (int64_t)R + 2;
     // The kernel that can read the sketch holds more registers, so fewer rows are resident per compute unit, and
-    // one launch serves the whole batch: it takes over only when most rows of the batch are better off with the
-    // sketch than with the cache.  Rows measure their share of cache hits in iteration kMemoDecide and those
-    // below the sketch's break-even share are counted on the device; the host reads the count at its next
-    // progress check.  If they are the majority, the break-even share of the sketch becomes the one that rows
-    // apply (rows below it leave the cache alone and use the sketch, the others keep the cache); otherwise the
-    // batch goes on as it would without a sketch.  Without a cache every row uses the sketch from the start.
+    // one launch serves the whole batch: it takes over only when most rows of the batch would rather use the
+    // sketch than the cache.  Rows find that out in iteration kMemoDecide and are counted on the device; the
+    // host reads the count at its next progress check.  In the other kernel a row that prefers the sketch goes
+    // on as it would without one.  Without a cache every row uses the sketch from the start.
     const uint8_t *sketch_table = step.sketch;
-    int sketch_rows_known = (sketch_table && !step.memo) ? 1 : -1;
+    int sketch_rows = sketch_from_start ? (int)p->n_rows : 0;
     int64_t t = 0;
     for (;;) {
         for (int r = 0; r < R; ++r) {
@@ -1284,7 +1324,7 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
             a.iter = (int)t;
             if (use_fused) {
                 step.m = a;
-                step.sketch = sketch_rows_known > 0 ? sketch_table : nullptr;
+                step.sketch = 2 * (int64_t)sketch_rows >= p->n_rows ? sketch_table : nullptr;
                 rc = launch_step_by_dim(step, aligned, merge_threads == 128 ? 128 : 256, smem, st);
                 if (rc < 0) return rc;
                 if (prof) VL_HIP(hipEventRecord(ev[3 * r + 1], st));
@@ -1308,14 +1348,9 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
         }
         int changed = 0;
         VL_HIP(hipMemcpyAsync(&changed, &ctrl->changed[(t / R) & 63], sizeof(int), hipMemcpyDeviceToHost, st));
-        const bool ask_dropped = sketch_table && sketch_rows_known < 0 && t >= kMemoDecide;
-        if (ask_dropped)
-            VL_HIP(hipMemcpyAsync(&sketch_rows_known, &ctrl->cache_dropped, sizeof(int), hipMemcpyDeviceToHost, st));
+        if (sketch_table && t >= kMemoDecide)
+            VL_HIP(hipMemcpyAsync(&sketch_rows, &ctrl->sketch_rows, sizeof(int), hipMemcpyDeviceToHost, st));
         VL_HIP(hipStreamSynchronize(st));
-        if (ask_dropped) {
-            if (2 * (int64_t)sketch_rows_known >= p->n_rows) step.memo_min_rate = step.sketch_min_rate;
-            else sketch_rows_known = 0;
-        }
         if (prof) {
             for (int r = 0; r < R; ++r) {
                 float ms = 0;

@@ -8,7 +8,7 @@
 //                 that is empty in every row (utils.py:63-66) because rows are
 //                 kept sorted
 //   changed[64] - ring of "some row changed" flags, one per checking iteration
-//   cache_dropped - how many rows gave up the per-row distance cache when they measured it
+//   sketch_rows - how many rows currently use the 8-bit sketch (they opt in once and may opt out once)
 #pragma once
 #include "vl_common.h"
 
@@ -19,7 +19,7 @@ struct BeamCtrl {
     int ended_after;  // iterations run when stop was set (for callers that enqueue a fixed number of launches)
     int first[3];
     int changed[64];
-    int cache_dropped;  // rows that measured their share of cache hits and left the distance cache alone
+    int sketch_rows;    // rows that currently look at their candidates through the 8-bit sketch first
     // profiling only, striped by workgroup so that the atomic adds do not queue up on one address:
     unsigned long long evals[kBeamStripes];   // candidate rows actually fetched
     unsigned long long wanted[kBeamStripes];  // candidate distances asked for (fetched or served by the cache)
