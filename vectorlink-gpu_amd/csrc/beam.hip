@@ -389,6 +389,27 @@ struct NoCount {
     __device__ __forceinline__ void operator()(int) const {}
 };
 
+// The fused step's, in the iteration in which a row measures its share of cache hits (word: the row's word of
+// the memo_rate array, else null; hits / asked: the row's counts in LDS).  A row would rather use the sketch than
+// the cache when few of its candidates repeat (its share of hits is below the sketch's break-even share) AND
+// few of them matter: the merge phase keeps the candidates below the queues' last slots, which are the ones a
+// sketched row has to evaluate exactly anyway - if that is more than a quarter of them (a row searching real
+// neighbour lists), the sketch saves nothing.  Every member is uniform over the workgroup.
+struct KeptCount {
+    int32_t *word;
+    int *sketch_rows;
+    const int *hits, *asked;
+    int min_rate, m;
+    __device__ __forceinline__ void operator()(int n_kept) const {
+        if (!word || threadIdx.x != 0) return;
+        const int rate = *asked > 0 ? (*hits * 256) / *asked : 256;
+        if (rate < min_rate && 4 * n_kept < m) {
+            *word = rate | (1 << 16);
+            atomicAdd(sketch_rows, 1);
+        }
+    }
+};
+
 template <int THREADS, bool FUSED, class Refine = NoRefine, class Kept = NoCount>
 __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *smem, RowState pre = RowState{0, 0},
                                           Refine refine = Refine(), Kept kept = Kept()) {
@@ -705,7 +726,7 @@ constexpr int kPreQ = 2, kPreV = 2, kPreS = 4;
 // candidates from a quarter of the bytes, then exact distances for the few whose lower bound is not above
 // every threshold that decides what the merge phase keeps.
 template <int CPL, int LPR, int U, bool GENERIC, int THREADS, int SCPL = 0, int SLPR = 64, int SU = 1>
-__global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
+__device__ __forceinline__ void beam_step_body(const StepArgs &s) {
     extern __shared__ __align__(16) unsigned char smem[];
     const MergeArgs &a = s.m;
     BeamCtrl *c = a.ctrl;
@@ -887,32 +908,21 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
         atomicAdd(&probe_hits_s, n_wanted - n_fetched);
     }
     __syncthreads();
-    int measured_rate = 256;
-    if (resample) {
-        measured_rate = probe_asked_s > 0 ? (probe_hits_s * 256) / probe_asked_s : 256;
-        if (tid == 0) s.memo_rate[row] = measured_rate;
-    }
-    // A row would rather use the sketch than the cache when few of its candidates repeat (its share of cache
-    // hits is below the sketch's break-even share) AND few of them matter: the merge phase keeps the candidates
-    // below the queues' last slots, which are the ones a sketched row has to evaluate exactly anyway - if that
-    // is more than a quarter of them (a row searching real neighbour lists), the sketch saves nothing.
-    auto kept = [&](int n_kept) {
-        if (resample && tid == 0 && measured_rate < s.sketch_min_rate && 4 * n_kept < a.m) {
-            s.memo_rate[row] = measured_rate | (1 << 16);
-            atomicAdd(&c->sketch_rows, 1);
-        }
-    };
+    if (resample && tid == 0) s.memo_rate[row] = probe_asked_s > 0 ? (probe_hits_s * 256) / probe_asked_s : 256;
+    const KeptCount kept{resample ? s.memo_rate + row : nullptr, &c->sketch_rows, &probe_hits_s, &probe_asked_s,
+                         s.sketch_min_rate, a.m};
     // ---- merge: ann.py:75-88 ----
     if constexpr (SCPL > 0) {
         // A sketched row knows every candidate distance only as lo <= d <= hi (ld holds lo, le holds hi).
         // What the merge phase keeps of the candidates: keys below the search queue's last slot (ws),
         // unvisited keys below the visit queue's last live slot (wv), and the Vt smallest distinct
-        // unvisited keys above wv.  Let tv be the Vt-th smallest hi among the distinct unvisited candidates
-        // that are certainly above wv (lo > wv): Vt candidates are then known to be at most tv, so a
-        // candidate with lo > tv is not one of the Vt smallest.  Hence a candidate whose lo is above ws, and
-        // which is visited or has lo above both wv and tv, cannot enter either queue and is dropped; all
-        // others are evaluated exactly, by the same code and in the same order as an unsketched row's.
-        // Comparisons are written so that a NaN bound counts as "evaluate".
+        // unvisited keys above wv.  Take any Vt distinct unvisited candidates that are certainly above wv
+        // (lo > wv) - those with the smallest hi, the likely winners - evaluate them, and let tv be the
+        // largest of their distances: Vt candidates are then known to be at most tv, so a candidate with
+        // lo > tv is not one of the Vt smallest.  Hence a candidate whose lo is above ws, and which is
+        // visited or has lo above both wv and tv, cannot enter either queue and is dropped; all others are
+        // evaluated exactly, by the same code and in the same order as an unsketched row's, in two rounds
+        // (the second one needs tv).  Comparisons are written so that a NaN bound counts as "evaluate".
         auto refine = [&](const int32_t *seen_b, int cnt, bool seen_full, uint64_t ws, uint64_t wv, uint8_t *flags,
                           uint64_t *red) {
             if (!sketching) return;  // uniform over the workgroup
@@ -932,7 +942,9 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
                 }
                 flags[i] = f;
             }
-            float tv = -1.0f;
+            // The Vt distinct candidates with the smallest upper bounds among those certainly above wv
+            // (bit 8), found one block-wide minimum at a time; fewer than Vt of them: every one may be taken.
+            bool all_rest = false;
             if (!seen_full) {
                 uint64_t last = 0ull;
                 for (int r = 0; r < a.Vt; ++r) {
@@ -943,27 +955,54 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
                         if ((r == 0 || k > last) && k < mine) mine = k;
                     }
                     const uint64_t mn = block_min_key(mine, red, r);
-                    if (mn == kPadKey) {  // fewer than Vt such candidates: every one of them may be taken
-                        tv = __builtin_inff();
+                    if (mn == kPadKey) {
+                        all_rest = true;
                         break;
                     }
                     last = mn;
-                    tv = vl_key_dist(mn);
+                    for (int i = tid; i < a.m; i += THREADS)
+                        if ((flags[i] & 2) && vl_make_key(li[i], le[i]) == mn) flags[i] |= 8;
                 }
             }
             int n_exact = 0, n_real = 0;
+            // first round: everything below a queue's last slot, and those Vt candidates
             for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
                 const int slot = c0 + lane;
                 const bool has = slot < a.m;
                 const int32_t cid = has ? li[slot] : VL_MAXINT;
                 const uint8_t f = has ? flags[slot] : 0;
-                const bool ok = (f & 4) || ((f & 2) && !(ld[slot] > tv));
-                if (has && cid != VL_MAXINT && !ok) {
+                const bool ok = (f & (4 | 8)) || (all_rest && (f & 2));
+                if (ok) flags[slot] = f | 16;  // its distance is exact from here on
+                n_exact += __popcll(__ballot(ok));
+                n_real += __popcll(__ballot(cid != VL_MAXINT));
+                wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0, nullptr, 0, false);
+            }
+            __syncthreads();
+            // tv: the largest exact distance of those Vt candidates.  Vt distinct unvisited candidates above wv
+            // are at most tv, so a candidate whose lower bound is above tv is not one of the Vt smallest.
+            float tv = -1.0f;
+            if (!seen_full && !all_rest) {
+                uint64_t mine = kPadKey;
+                for (int i = tid; i < a.m; i += THREADS)
+                    if (flags[i] & 8) {
+                        const uint64_t k = ~(uint64_t)vl_float_key(ld[i]);
+                        mine = k < mine ? k : mine;
+                    }
+                const uint64_t mn = block_min_key(mine, red, a.Vt);
+                tv = mn == kPadKey ? -1.0f : vl_key_float((uint32_t)~mn);
+            }
+            // second round: the candidates above wv that may still be among the Vt smallest
+            for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
+                const int slot = c0 + lane;
+                const bool has = slot < a.m;
+                const int32_t cid = has ? li[slot] : VL_MAXINT;
+                const uint8_t f = has ? flags[slot] : 0;
+                const bool ok = (f & 2) && !(f & 16) && !(ld[slot] > tv);
+                if (has && cid != VL_MAXINT && !ok && !(f & 16)) {
                     li[slot] = VL_MAXINT;
                     ld[slot] = VL_MAXFLOAT;
                 }
                 n_exact += __popcll(__ballot(ok));
-                n_real += __popcll(__ballot(cid != VL_MAXINT));
                 wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0, nullptr, 0, false);
             }
             if (s.count_evals && lane == 0 && n_exact)
@@ -993,18 +1032,44 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
     }
 }
 
-template <int CPL, int LPR, int U, bool GENERIC, int SCPL = 0, int SLPR = 64, int SU = 1>
+template <int CPL, int LPR, int U, bool GENERIC, int THREADS>
+__global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
+    beam_step_body<CPL, LPR, U, GENERIC, THREADS>(s);
+}
+
+// The same step for rows that may use the sketch.  WPE: wavefronts per SIMD the compiler is asked to leave room
+// for.  The sketch's copy of the query row takes 16 registers per chunk and lane, and a row's phases (sketch
+// pass, two rounds of exact rows, merge) each wait on memory, so residency is worth a few spilled registers:
+// measured at 768 and 384 columns, five wavefronts per SIMD with two loads in flight beat three wavefronts
+// with four (0.84 -> 0.75 ms and 0.61 -> 0.43 ms per launch).
+template <int CPL, int LPR, int U, int THREADS, int SCPL, int SLPR, int SU, int WPE>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPE)))
+void beam_step_sketch_kernel(StepArgs s) {
+    beam_step_body<CPL, LPR, U, false, THREADS, SCPL, SLPR, SU>(s);
+}
+
+template <int CPL, int LPR, int U, bool GENERIC, int SCPL = 0, int SLPR = 64, int SU = 1, int WPE = 4>
 void launch_step(const StepArgs &s, int threads, size_t smem, hipStream_t st) {
     dim3 grid((unsigned)s.m.n_rows);
     if constexpr (SCPL > 0) {
         if (!s.sketch) return launch_step<CPL, LPR, U, GENERIC>(s, threads, smem, st);
     }
-    if (threads == 128) {
-        auto kernel = beam_step_kernel<CPL, LPR, U, GENERIC, 128, SCPL, SLPR, SU>;
-        if (vl_allow_lds(kernel, smem) != hipSuccess) return;  // seen by the launch check
+    if constexpr (SCPL > 0) {
+        if (threads == 128) {
+            auto kernel = beam_step_sketch_kernel<CPL, LPR, U, 128, SCPL, SLPR, SU, WPE>;
+            if (vl_allow_lds(kernel, smem) != hipSuccess) return;  // seen by the launch check
+            hipLaunchKernelGGL(kernel, grid, dim3(128), smem, st, s);
+        } else {
+            auto kernel = beam_step_sketch_kernel<CPL, LPR, U, 256, SCPL, SLPR, SU, WPE>;
+            if (vl_allow_lds(kernel, smem) != hipSuccess) return;
+            hipLaunchKernelGGL(kernel, grid, dim3(256), smem, st, s);
+        }
+    } else if (threads == 128) {
+        auto kernel = beam_step_kernel<CPL, LPR, U, GENERIC, 128>;
+        if (vl_allow_lds(kernel, smem) != hipSuccess) return;
         hipLaunchKernelGGL(kernel, grid, dim3(128), smem, st, s);
     } else {
-        auto kernel = beam_step_kernel<CPL, LPR, U, GENERIC, 256, SCPL, SLPR, SU>;
+        auto kernel = beam_step_kernel<CPL, LPR, U, GENERIC, 256>;
         if (vl_allow_lds(kernel, smem) != hipSuccess) return;
         hipLaunchKernelGGL(kernel, grid, dim3(256), smem, st, s);
     }
@@ -1020,24 +1085,25 @@ int dist_variant() {
     return v;
 }
 
-// The last three numbers are the sketch's lane shape for rows of that size: a sketch row has a quarter of
-// the chunks, so a quarter of the lanes (or of the chunks per lane) covers it.
+// The numbers after `false` are the sketch's lane shape for rows of that size (chunks per lane, lanes per row,
+// loads in flight) and the wavefronts per SIMD asked for: a sketch row has a quarter of the chunks, so a quarter
+// of the lanes (or of the chunks per lane) covers it.
 int launch_step_by_dim(const StepArgs &s, bool aligned, int threads, size_t smem, hipStream_t st) {
     const int nchunks = s.nchunks;
     const int variant = dist_variant();
     if (!aligned || nchunks > 512) launch_step<1, 64, 1, true>(s, threads, smem, st);
-    else if (nchunks <= 16) launch_step<1, 16, 8, false, 1, 8, 8>(s, threads, smem, st);
+    else if (nchunks <= 16) launch_step<1, 16, 8, false, 1, 8, 4, 5>(s, threads, smem, st);
     else if (nchunks <= 32 && variant == 1) launch_step<1, 32, 8, false>(s, threads, smem, st);
-    else if (nchunks <= 32) launch_step<2, 16, 4, false, 1, 8, 8>(s, threads, smem, st);
-    else if (nchunks <= 64) launch_step<1, 64, 8, false, 2, 8, 4>(s, threads, smem, st);
-    else if (nchunks <= 96 && variant != 1) launch_step<3, 32, 4, false, 3, 8, 4>(s, threads, smem, st);
-    else if (nchunks <= 128) launch_step<2, 64, 8, false, 2, 16, 4>(s, threads, smem, st);
-    else if (nchunks <= 192) launch_step<3, 64, 4, false, 3, 16, 4>(s, threads, smem, st);
-    else if (nchunks <= 256) launch_step<4, 64, 4, false, 4, 16, 2>(s, threads, smem, st);
-    else if (nchunks <= 320) launch_step<5, 64, 2, false, 3, 32, 4>(s, threads, smem, st);
-    else if (nchunks <= 384) launch_step<6, 64, 2, false, 3, 32, 4>(s, threads, smem, st);
-    else if (nchunks <= 448) launch_step<7, 64, 2, false, 4, 32, 2>(s, threads, smem, st);
-    else launch_step<8, 64, 2, false, 4, 32, 2>(s, threads, smem, st);
+    else if (nchunks <= 32) launch_step<2, 16, 4, false, 1, 8, 4, 5>(s, threads, smem, st);
+    else if (nchunks <= 64) launch_step<1, 64, 8, false, 2, 8, 2, 5>(s, threads, smem, st);
+    else if (nchunks <= 96 && variant != 1) launch_step<3, 32, 4, false, 3, 8, 2, 5>(s, threads, smem, st);
+    else if (nchunks <= 128) launch_step<2, 64, 8, false, 2, 16, 2, 5>(s, threads, smem, st);
+    else if (nchunks <= 192) launch_step<3, 64, 4, false, 3, 16, 2, 5>(s, threads, smem, st);
+    else if (nchunks <= 256) launch_step<4, 64, 4, false, 4, 16, 2, 4>(s, threads, smem, st);
+    else if (nchunks <= 320) launch_step<5, 64, 2, false, 3, 32, 2, 5>(s, threads, smem, st);
+    else if (nchunks <= 384) launch_step<6, 64, 2, false, 3, 32, 2, 5>(s, threads, smem, st);
+    else if (nchunks <= 448) launch_step<7, 64, 2, false, 4, 32, 2, 4>(s, threads, smem, st);
+    else launch_step<8, 64, 2, false, 4, 32, 2, 4>(s, threads, smem, st);
     VL_LAUNCH_CHECK("beam_step_kernel");
     return VL_OK;
 }
