@@ -228,11 +228,12 @@ int64_t vl_closest_vectors(const vl_beam_params *p,
  * The reference evaluates every candidate distance of an iteration in full
  * (cuda_search_from_seeds_kernel, kernels.py:204-257) although a row keeps a
  * handful of its hundreds of candidates.  A sketch row holds the vector rounded
- * to 8 bits per element with one scale per row (dim bytes, padded to a multiple
- * of 16) and a 16-byte tail: float scale, float bound on the 2-norm of what the
- * rounding moved, float bound on the row's 2-norm, float 0.  With it a dot
- * product is known to within ||q|| x that bound (Cauchy-Schwarz) from a quarter
- * of the bytes.  vl_closest_vectors_with_sketch uses those bounds ONLY to decide
+ * to 8 bits per element with one scale per row (dim int8 values round(v / scale),
+ * scale = max |v| / 127, padded with zeros to a multiple of 16) and a 16-byte
+ * tail: float scale, float bound on the 2-norm of what the rounding moved, float
+ * bound on the row's 2-norm, float 0.  With it a dot product is known to within
+ * ||q|| x that bound (Cauchy-Schwarz) from a quarter of the bytes, by integer
+ * arithmetic (the query row is rounded to 15 bits, which the bound accounts for).  vl_closest_vectors_with_sketch uses those bounds ONLY to decide
  * which candidate rows to fetch: a candidate whose lower bound is above the last
  * slot of the search queue and, when it is unvisited, above the last live slot
  * of the visit queue and above the parallel_visit_count-th smallest upper bound

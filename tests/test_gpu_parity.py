@@ -1012,7 +1012,7 @@ def test_queues_beyond_64_kib_of_lds():
 def test_sketch_rows_bound_every_dot_product(dim):
     """build_sketch: the bytes are the row rounded to 8 bits under the row's own scale, and the tail's two
     bounds hold against float64 - the 2-norm of what the rounding moved, and the row's 2-norm.  Then, for
-    random queries, |<q, v> - scale * <q, u - 128>| <= ||q|| * bound, which is what the search relies on."""
+    random queries, |<q, v> - scale * <q, u>| <= ||q|| * bound, which is what the search relies on."""
     say(f"sketch rows dim={dim}")
     from vectorlink_gpu.kernels import build_sketch, sketch_row_bytes
 
@@ -1031,10 +1031,10 @@ def test_sketch_rows_bound_every_dot_product(dim):
     t = host(build_sketch(dev(v)))
     assert t.shape == (n, rb)
     pad = rb - 16
-    u = t[:, :dim].astype(np.float64) - 128.0
+    u = t[:, :dim].view(np.int8).astype(np.float64)
     tail = t[:, pad:].copy().view(np.float32)
     scale, resid, norm = tail[:, 0].astype(np.float64), tail[:, 1].astype(np.float64), tail[:, 2].astype(np.float64)
-    assert np.all(t[:, dim:pad] == 128) and np.all(tail[:, 3] == 0)
+    assert np.all(t[:, dim:pad] == 0) and np.all(tail[:, 3] == 0)
     bad = ~np.isfinite(v).all(axis=1)
     assert np.all(np.isinf(resid[bad])) and np.all(np.isinf(norm[bad]))
     ok = ~bad

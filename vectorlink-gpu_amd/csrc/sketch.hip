@@ -51,7 +51,7 @@ __global__ __launch_bounds__(256) void sketch_build_kernel(const float *__restri
                 r2 = __builtin_fmaf(e, e, r2);
                 n2 = __builtin_fmaf(x, x, n2);
             }
-            word |= (uint32_t)((int)qv + 128) << (8 * k);
+            word |= (uint32_t)((int)qv & 0xff) << (8 * k);
         }
         reinterpret_cast<uint32_t *>(out)[g] = word;
     }

@@ -6,16 +6,19 @@
 // for a quarter of the memory traffic.  A sketch row holds the vector rounded to 8 bits per element
 // with one scale per row, and how far that rounding moved the vector:
 //
-//   bytes [0, dim)            u_j = round(v_j / scale) + 128, scale = max_j |v_j| / 127
-//   bytes [dim, pad16(dim))   128 (a zero element)
-//   tail, 16 bytes            float scale; float resid >= ||v - scale (u - 128)||_2;
-//                             float norm >= ||v||_2; float 0
+//   bytes [0, dim)            int8 u_j = round(v_j / scale), scale = max_j |v_j| / 127
+//   bytes [dim, pad16(dim))   0
+//   tail, 16 bytes            float scale; float resid >= ||v - scale u||_2; float norm >= ||v||_2; float 0
 //
-// For a query q, s^ = scale * sum_j q_j (u_j - 128) differs from the dot product <q, v> by at most
-// ||q||_2 * resid (Cauchy-Schwarz).  Adding the rounding of the two float32 summations involved (this
-// one, and the one the exact kernel performs: at most (dim + 16) * 2^-24 times the sum of the absolute
-// values of their terms) gives an eps with |s^ - s| <= eps for the very float s the exact kernel
-// computes, and because the map from s to the clamped cosine distance is monotone, rounding included,
+// The query row is rounded too, to 15 bits per element (Q_j = round(q_j / qscale) = 128 qh_j + ql_j with
+// two int8 digits, qscale = max_j |q_j| / 16256), so that the sum is integer work, four elements per
+// v_dot4_i32_i8 and exact: s^ = scale * qscale * sum_j Q_j u_j.  It differs from the dot product <q, v> by
+//   <q, v - v^> + <q - q^, v^>,   at most ||q|| resid + ||q - q^|| (norm + resid)   (Cauchy-Schwarz),
+// with ||q - q^|| <= qscale / 2 * sqrt(dim).  Adding the rounding of the few float operations that turn
+// the integer sums into s^, and of the float32 summation the exact kernel performs (at most
+// (dim + 16) * 2^-24 times the sum of the absolute values of its terms), gives an eps with
+// |s^ - s| <= eps for the very float s the exact kernel computes, and because the map from s to the
+// clamped cosine distance is monotone, rounding included,
 // lo = distance(s^ + eps) <= exact distance <= hi = distance(s^ - eps).  Nothing that is returned to
 // a caller is ever computed from a sketch: the bounds only decide which candidates are evaluated
 // exactly (dist_device.h) and which provably cannot enter a queue.
@@ -24,12 +27,6 @@
 
 __host__ __device__ inline int64_t sketch_data_chunks(int64_t dim) { return (dim + 15) / 16; }
 __host__ __device__ inline int64_t sketch_row_bytes(int64_t dim) { return sketch_data_chunks(dim) * 16 + 16; }
-
-// Byte K of a word as a float (the compiler has one instruction for it: v_cvt_f32_ubyteK).
-template <int K>
-__device__ __forceinline__ float byte_as_float(unsigned w) {
-    return (float)((w >> (8 * K)) & 0xffu);
-}
 
 // Sum over a group of N neighbouring lanes, left in the group's first lane (other lanes end with
 // values nobody uses).  Same moves as fold_group, for groups of 8 lanes as well.
@@ -44,45 +41,62 @@ __device__ __forceinline__ float fold_lanes(float acc) {
 }
 
 // The query row as the lanes of a group hold it for the sketch: 16-element chunk c belongs to lane
-// c mod SLPR of the group, and what the bound needs of the row as a whole.
+// c mod SLPR of the group; four elements per word, high and low digit apart.
 template <int SCPL>
 struct SketchQuery {
-    float q[SCPL][16];
-    float sum128;  // 128 * sum_j q_j : what the +128 offset of the bytes adds to sum_j q_j u_j
+    int qh[SCPL][4], ql[SCPL][4];
+    float qscale;  // the step of the rounded query
     float norm2;   // ||q||_2
-    float roundc;  // per unit of scale: bound on the rounding of sum_j q_j u_j - 128 sum_j q_j
+    float qerr;    // >= ||q - q^||_2
     float exactc;  // per unit of ||v||_2: bound on the rounding of the exact kernel's dot product
 };
 
 template <int SCPL, int SLPR>
 __device__ __forceinline__ void sketch_query_load(SketchQuery<SCPL> &sq, const float *__restrict__ q_row, int dim) {
     const int lig = (threadIdx.x & (kWave - 1)) % SLPR;
-    float s = 0.f, a = 0.f, n = 0.f;
+    float4 x[SCPL][4];
+    float mx = 0.f, n = 0.f;
 #pragma unroll
     for (int i = 0; i < SCPL; ++i) {
         const int c = lig + SLPR * i;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
             const int j = 16 * c + 4 * w;  // dim is a multiple of 4 on this path
-            const float4 x = j < dim ? *reinterpret_cast<const float4 *>(q_row + j) : make_float4(0.f, 0.f, 0.f, 0.f);
-            sq.q[i][4 * w + 0] = x.x; sq.q[i][4 * w + 1] = x.y; sq.q[i][4 * w + 2] = x.z; sq.q[i][4 * w + 3] = x.w;
-            s += (x.x + x.y) + (x.z + x.w);
-            a += (__builtin_fabsf(x.x) + __builtin_fabsf(x.y)) + (__builtin_fabsf(x.z) + __builtin_fabsf(x.w));
-            n = __builtin_fmaf(x.x, x.x, n); n = __builtin_fmaf(x.y, x.y, n);
-            n = __builtin_fmaf(x.z, x.z, n); n = __builtin_fmaf(x.w, x.w, n);
+            x[i][w] = j < dim ? *reinterpret_cast<const float4 *>(q_row + j) : make_float4(0.f, 0.f, 0.f, 0.f);
+            mx = fmaxf(fmaxf(mx, fmaxf(__builtin_fabsf(x[i][w].x), __builtin_fabsf(x[i][w].y))),
+                       fmaxf(__builtin_fabsf(x[i][w].z), __builtin_fabsf(x[i][w].w)));
+            n = __builtin_fmaf(x[i][w].x, x[i][w].x, n); n = __builtin_fmaf(x[i][w].y, x[i][w].y, n);
+            n = __builtin_fmaf(x[i][w].z, x[i][w].z, n); n = __builtin_fmaf(x[i][w].w, x[i][w].w, n);
         }
     }
 #pragma unroll
     for (int h = SLPR / 2; h >= 1; h >>= 1) {  // every lane of the group ends with the totals
-        s += __shfl_xor(s, h);
-        a += __shfl_xor(a, h);
+        mx = fmaxf(mx, __shfl_xor(mx, h));
         n += __shfl_xor(n, h);
     }
-    const float u = (float)(dim + 16) * 5.9604645e-8f;  // (dim + 16) * 2^-24
-    sq.sum128 = 128.0f * s;
-    sq.norm2 = __builtin_sqrtf(n);
-    sq.roundc = u * 383.0f * a;  // terms |q_j| * u_j <= 255 |q_j| of the one sum, 128 |q_j| of the other
-    sq.exactc = u * sq.norm2;    // terms |q_j v_j| sum to at most ||q||_2 ||v||_2
+    // a row of zeros, of denormals, or one with a NaN: rounded to zero, and the bound is the row's whole length
+    const bool tiny = !(mx > 1e-30f);
+    const float inv = tiny ? 0.f : 16256.0f / mx;
+    auto digits = [&](float v, int &hi, int &lo) {
+        const int q = (int)fminf(fmaxf(rintf(v * inv), -16256.0f), 16256.0f);
+        lo = ((q + 64) & 127) - 64;   // [-64, 63]
+        hi = (q - lo) >> 7;           // [-127, 127], q = 128 hi + lo
+    };
+#pragma unroll
+    for (int i = 0; i < SCPL; ++i)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            int h0, l0, h1, l1, h2, l2, h3, l3;
+            digits(x[i][w].x, h0, l0); digits(x[i][w].y, h1, l1); digits(x[i][w].z, h2, l2); digits(x[i][w].w, h3, l3);
+            sq.qh[i][w] = (h0 & 0xff) | ((h1 & 0xff) << 8) | ((h2 & 0xff) << 16) | ((h3 & 0xff) << 24);
+            sq.ql[i][w] = (l0 & 0xff) | ((l1 & 0xff) << 8) | ((l2 & 0xff) << 16) | ((l3 & 0xff) << 24);
+        }
+    sq.qscale = mx / 16256.0f;
+    sq.norm2 = __builtin_sqrtf(n) * 1.001f;
+    // an element moves by at most half a step (0.51: v * inv and the step itself are rounded floats); a NaN or an
+    // infinity in the query makes the bound a NaN or an infinity, which the callers read as "evaluate"
+    sq.qerr = tiny ? sq.norm2 : 0.51f * sq.qscale * __builtin_sqrtf((float)(16 * SCPL * SLPR));
+    sq.exactc = (float)(dim + 16) * 5.9604645e-8f * sq.norm2;  // terms |q_j v_j| sum to at most ||q||_2 ||v||_2
 }
 
 // One wavefront: lane j holds candidate id `my_id` (valid when `ok`); the bounds of its distance to
@@ -127,23 +141,25 @@ __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const u
         }
 #pragma unroll
         for (int u = 0; u < SU; ++u) {
-            float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+            int sh = 0, sl = 0;
 #pragma unroll
             for (int i = 0; i < SCPL; ++i) {
-                const unsigned w[4] = {r[u][i].x, r[u][i].y, r[u][i].z, r[u][i].w};
+                const int w[4] = {(int)r[u][i].x, (int)r[u][i].y, (int)r[u][i].z, (int)r[u][i].w};
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    a0 = __builtin_fmaf(byte_as_float<0>(w[k]), sq.q[i][4 * k + 0], a0);
-                    a1 = __builtin_fmaf(byte_as_float<1>(w[k]), sq.q[i][4 * k + 1], a1);
-                    a2 = __builtin_fmaf(byte_as_float<2>(w[k]), sq.q[i][4 * k + 2], a2);
-                    a3 = __builtin_fmaf(byte_as_float<3>(w[k]), sq.q[i][4 * k + 3], a3);
+                    sh = __builtin_amdgcn_sdot4(w[k], sq.qh[i][k], sh, false);
+                    sl = __builtin_amdgcn_sdot4(w[k], sq.ql[i][k], sl, false);
                 }
             }
-            float acc = fold_lanes<SLPR>((a0 + a1) + (a2 + a3));
+            // a lane's two sums are below 2^24 (at most 64 elements of 127 * 127 each), so they convert exactly
+            const float acc = fold_lanes<SLPR>(__builtin_fmaf(128.0f, (float)sh, (float)sl));
             if (lig == 0 && mysrc[u] >= 0) {
                 const float scale = tail[u].x, resid = tail[u].y, norm = tail[u].z;
-                const float s_hat = scale * (acc - sq.sum128);
-                const float eps = (sq.norm2 * resid + scale * sq.roundc + sq.exactc * norm) * 1.0001f + 2e-7f;
+                const float s_hat = (scale * sq.qscale) * acc;
+                // 4e-6: the integer sums are exact, the float operations that combine them (one fused
+                // multiply-add per lane, up to six adds across lanes, two products) each round by 2^-24 of at most
+                // ||q^|| ||v^||
+                const float eps = (sq.norm2 * resid + (sq.qerr + 4e-6f * sq.norm2) * (norm + resid) + sq.exactc * norm) * 1.0001f + 2e-7f;
                 out_lo[mysrc[u]] = clamp_distance(s_hat + eps);
                 out_hi[mysrc[u]] = clamp_distance(s_hat - eps);
             }
