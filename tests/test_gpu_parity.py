@@ -1128,3 +1128,25 @@ def test_closest_vectors_with_sketch(n, dim, beam, bqf, pv, vqf, ef, ra, cache):
         # with the cache, rows switch only if few of their candidates repeat and few of them matter
     else:
         assert sketched == 0
+
+
+def test_build_with_and_without_the_sketch():
+    """ANN builds the sketch for rows of 1 KiB and more and searches the initial circulant graph through it
+    (no distance cache in that loop); sketch=False builds as before.  Both give the oracle's graph."""
+    say("build with and without the sketch, n=3000 dim=256")
+    from vectorlink_gpu import ANN
+    from vectorlink_gpu.ann import GraphBuild
+
+    rng = np.random.default_rng(256)
+    n, dim = 3000, 256
+    centres = rng.standard_normal((30, dim)).astype(np.float32)
+    v = centres[rng.integers(0, 30, n)] + 0.15 * rng.standard_normal((n, dim)).astype(np.float32)
+    v = (v / np.linalg.norm(v, axis=1, keepdims=True)).astype(np.float32)
+    kw = dict(beam_size=16, beam_queue_factor=2, batch_size=800, optimization_loops=2)
+    (wb, wd) = orc.generate_ann(v, cfg(**kw))
+    gv = dev(v)
+    assert GraphBuild(gv, cfg(**kw)).sketch is not None and GraphBuild(gv, cfg(sketch=False, **kw)).sketch is None
+    for sketch in (True, False):
+        ann = ANN(gv, sketch=sketch, **kw)
+        assert np.array_equal(host(ann.beams), wb), sketch
+        assert np.array_equal(bits(host(ann.distances)), bits(wd)), sketch

@@ -510,6 +510,7 @@ class ANN:
         metric: str = "cosine",
         concurrent_batches: int = 4,
         seed_dims: Optional[int] = None,
+        sketch: bool = True,
     ):
         """seeding / entry_points are additions: "circulant" seeds searches as the
         reference does; "dense" seeds them from the nearest of `entry_points`
@@ -523,7 +524,9 @@ class ANN:
         that the build keeps in flight, each on its own stream and host thread; the
         graph does not depend on it.  metric is an addition too: "cosine" is the reference's distance; "l2" builds
         and searches by squared Euclidean distance (rows need not be unit length);
-        dense seeding and recall_at_k follow the metric."""
+        dense seeding and recall_at_k follow the metric.  sketch (an addition): the build keeps an
+        8-bit copy of rows of 1 KiB and more and lets searches of the initial graph decide from it
+        which candidate rows to fetch (kernels.build_sketch); the graph is the same either way."""
         assert prune in (True, False, "rank")
         nv.metric_code(metric)
         assert vectors.dim() == 2 and vectors.dtype == torch.float32
@@ -549,6 +552,8 @@ class ANN:
         }
         if metric != "cosine":
             self.configuration["metric"] = metric
+        if not sketch:
+            self.configuration["sketch"] = False
         if not vectors.is_cuda:
             vectors = vectors.to(DEVICE)
         self.vectors = vectors.contiguous()
