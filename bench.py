@@ -254,6 +254,9 @@ def main():
     ap.add_argument("--loops", type=int, default=3, help="optimisation loops of the build (the reference's default is 3)")
     ap.add_argument("--concurrent-batches", type=int, default=4,
                     help="batches of an optimisation loop kept in flight by the timed build (streams / host threads)")
+    ap.add_argument("--no-sketch", action="store_true",
+                    help="build without the 8-bit sketch of the vectors (every candidate row of the first loop is "
+                         "fetched whole, as before the sketch existed; the graph is the same)")
     ap.add_argument("--prune", choices=["reference", "rank", "none"], default="reference",
                     help="reference = prune_ between loops as the reference does (default); rank = detour-count "
                          "cut with reverse edges at the end (an addition); none = no pruning")
@@ -281,6 +284,8 @@ def main():
     cfg = dict(prune={"reference": True, "rank": "rank", "none": False}[args.prune], parallel_visit_count=4,
                visit_queue_factor=3, exclude_factor=5, optimization_loops=args.loops, batch_size=10_000,
                speculative_readahead=5, **kwargs)
+    if args.no_sketch:
+        cfg["sketch"] = False
     vectors = base.to(dev)
     qdev = queries.to(dev)
     torch.cuda.synchronize()
@@ -413,6 +418,9 @@ def main():
                    "optimization_loops": cfg["optimization_loops"], "parallel_visit_count": 4,
                    "prune": args.prune, "build_seeding": "circulant (reference)",
                    "concurrent_batches": args.concurrent_batches,
+                   "sketch": "8-bit sketch of the vectors decides which candidate rows the first loop fetches; "
+                             "graph bit-identical" if build.sketch is not None else "none",
+                   "sketch_bytes": int(build.sketch.numel()) if build.sketch is not None else 0,
                    "search_seeding": "dense, 32768 entry points", "queries": int(queries.shape[0])},
         "partial": False, "build_seconds": t_build, "build_steps": done,
         "steps_note": f"value = n / build_seconds over all {done} steps (hooks off); steps and ms_per_step describe "
