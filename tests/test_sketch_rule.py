@@ -12,10 +12,13 @@ M, F = orc.MAXINT, orc.MAXFLOAT
 
 
 def bounds_for(ids, d, slack, seed):
-    """lo <= d <= hi with a gap that depends on the id alone (as a sketch row's does), up to `slack` each side."""
+    """lo <= d <= hi with a gap of up to `slack` each side that depends on the id (as a sketch row's does) and,
+    a little, on the slot: copies of one id may carry different bounds (fresh from the sketch, or decoded from
+    the cache and a step wider)."""
     h = (ids.astype(np.int64) * 2654435761 + seed) % 1000003
-    below = (h % 997) / 997.0 * slack
-    above = ((h // 997) % 991) / 991.0 * slack
+    widen = 1.0 + 0.05 * (np.arange(ids.shape[0]) % 3)
+    below = (h % 997) / 997.0 * slack * widen
+    above = ((h // 997) % 991) / 991.0 * slack * widen
     lo = np.maximum(d - below, 0).astype(np.float32)
     hi = np.minimum(d + above, 1).astype(np.float32)
     lo[ids == M] = F
@@ -35,12 +38,14 @@ def drop_by_rule(ids, d, lo, hi, ws_d, wv_d, seen, vt):
         unseen = real & ~np.isin(ids, seen[seen != M])
         need |= unseen & ~(lo > wv_d)
         rest = unseen & (lo > wv_d)
-        keys = sorted({(float(hi[i]), int(ids[i])) for i in np.flatnonzero(rest)})
-        if len(keys) < vt:
+        first = []   # vt distinct ids, smallest (hi, id) first; every copy of a chosen id goes with it
+        for (_, cid) in sorted((float(hi[i]), int(ids[i])) for i in np.flatnonzero(rest)):
+            if cid not in first and len(first) < vt:
+                first.append(cid)
+        if len(first) < vt:
             need |= rest
         else:
-            first = {k[1] for k in keys[:vt]}
-            winners = rest & np.isin(ids, list(first))
+            winners = rest & np.isin(ids, first)
             tv = d[winners].max()
             need |= winners | (rest & ~(lo > tv))
     return need

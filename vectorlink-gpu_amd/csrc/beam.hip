@@ -384,35 +384,9 @@ struct NoRefine {
     __device__ __forceinline__ void operator()(const int32_t *, int, bool, uint64_t, uint64_t, uint8_t *, uint64_t *) const {}
 };
 
-// kept (fused step only): told how many candidates of the row the merge phase keeps for its queues.
-struct NoCount {
-    __device__ __forceinline__ void operator()(int) const {}
-};
-
-// The fused step's, in the iteration in which a row measures its share of cache hits (word: the row's word of
-// the memo_rate array, else null; hits / asked: the row's counts in LDS).  A row would rather use the sketch than
-// the cache when few of its candidates repeat (its share of hits is below the sketch's break-even share) AND
-// few of them matter: the merge phase keeps the candidates below the queues' last slots, which are the ones a
-// sketched row has to evaluate exactly anyway - if that is more than a quarter of them (a row searching real
-// neighbour lists), the sketch saves nothing.  Every member is uniform over the workgroup.
-struct KeptCount {
-    int32_t *word;
-    int *sketch_rows;
-    const int *hits, *asked;
-    int min_rate, m;
-    __device__ __forceinline__ void operator()(int n_kept) const {
-        if (!word || threadIdx.x != 0) return;
-        const int rate = *asked > 0 ? (*hits * 256) / *asked : 256;
-        if (rate < min_rate && 4 * n_kept < m) {
-            *word = rate | (1 << 16);
-            atomicAdd(sketch_rows, 1);
-        }
-    }
-};
-
-template <int THREADS, bool FUSED, class Refine = NoRefine, class Kept = NoCount>
+template <int THREADS, bool FUSED, class Refine = NoRefine>
 __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *smem, RowState pre = RowState{0, 0},
-                                          Refine refine = Refine(), Kept kept = Kept()) {
+                                          Refine refine = Refine()) {
     const int Pc = a.Pc;
     uint64_t *raw = reinterpret_cast<uint64_t *>(smem);  // candidate keys as they arrive
     uint64_t *uk = raw + Pc;                             // the candidates that can matter, then sorted
@@ -583,7 +557,6 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
         return (f & 1) || ((f & 2) && raw[i] <= sel_max);
     };
     const int n_u = block_compact(raw, a.m, uk, wanted, wave_cnt);
-    kept(n_u);
     int Pu = 2;
     while (Pu < n_u) Pu <<= 1;
     for (int i = n_u + threadIdx.x; i < Pu; i += blockDim.x) uk[i] = kPadKey;
@@ -698,7 +671,6 @@ struct StepArgs {
     int memo_shift;
     int32_t *memo_rate;   // per row: share (x 256) of the candidates of iteration kMemoDecide that were cached; bit 16: the row prefers the sketch
     int memo_min_rate;    // the cache stays in use only if that share is at least this (x 256)
-    int sketch_min_rate;  // rows whose share is below this (x 256) are counted in the control block (0: nobody counts)
     int count_evals;
     int l2;  // 0: cosine distance, 1: squared L2
     const uint8_t *sketch;     // 8-bit sketch of `vectors` (sketch_device.h), or null
@@ -798,7 +770,6 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
     if (memo_row && memo_rate < s.memo_min_rate) memo_row = nullptr;
     bool sketching = false;
     if constexpr (SCPL > 0) sketching = (memo_word >> 16) != 0;
-    if (sketching) memo_row = nullptr;
     const bool probing = memo_row != nullptr;
     if (tid < a.Vt) g_visit_s[tid] = my_visit;
     if (tid == 0) {
@@ -855,6 +826,7 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
     }
     int n_wanted = 0, n_fetched = 0, n_sketched = 0;  // counts of this wavefront
     float *le = reinterpret_cast<float *>(raw);                     // upper bounds (raw is filled in the merge phase)
+    uint8_t *xf = reinterpret_cast<uint8_t *>(exl + a.excl_cols);   // the merge phase's per-candidate flags; 16 = exact
     if constexpr (SCPL > 0) {
         if (sketching) {
             SketchQuery<SCPL> sq;
@@ -863,15 +835,36 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
                 if (c0 != wave * kWave) id = resolve(c0);
                 const int slot = c0 + lane;
                 const bool has = slot < a.m;
-                const bool ok = has && id != VL_MAXINT && id >= 0 && (int64_t)id < s.n_vectors;
+                bool ok = has && id != VL_MAXINT && id >= 0 && (int64_t)id < s.n_vectors;
                 if (has) {
                     li[slot] = ok ? id : VL_MAXINT;
                     if (!ok) ld[slot] = VL_MAXFLOAT;
+                    xf[slot] = 0;
                 }
-                if (s.count_evals) n_sketched += __popcll(__ballot(ok));
-                wave_sketch<SCPL, SLPR, SU>(sq, s.sketch, s.sketch_row_bytes, s.sketch_chunks, id, ok, ld + c0, le + c0);
+                if (s.count_evals || resample) n_wanted += __popcll(__ballot(ok));
+                // The cache serves two kinds of repeats: a candidate evaluated exactly before comes back with its
+                // distance, one that was only bounded comes back with its bounds (dist_device.h) - either way
+                // nothing is fetched for it now.
+                if (probing && ok) {
+                    const uint64_t e = memo_load(memo_row, s.memo_shift, id);
+                    if ((int32_t)((uint32_t)e & ~kMemoBounds) == id) {
+                        if ((uint32_t)e & kMemoBounds) {
+                            ld[slot] = memo_bound_lo(e);
+                            le[slot] = memo_bound_hi(e);
+                        } else {
+                            const float d = __builtin_bit_cast(float, (uint32_t)(e >> 32));
+                            ld[slot] = d;
+                            le[slot] = d;
+                            xf[slot] = 16;  // exact already
+                        }
+                        ok = false;
+                    }
+                }
+                if (s.count_evals || resample) n_sketched += __popcll(__ballot(ok));
+                wave_sketch<SCPL, SLPR, SU>(sq, s.sketch, s.sketch_row_bytes, s.sketch_chunks, id, ok, ld + c0, le + c0,
+                                            memo_row, s.memo_shift);
             }
-            n_wanted = n_sketched;
+            n_fetched = n_sketched;  // for the share of cache hits: what the cache did not answer
         }
     }
     for (int c0 = wave * kWave; c0 < a.m && !sketching; c0 += THREADS) {
@@ -900,7 +893,7 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
     if (s.count_evals && lane == 0) {
         const int stripe = (int)((blockIdx.x * (THREADS / kWave) + wave) & (kBeamStripes - 1));
         if (n_wanted) atomicAdd(&c->wanted[stripe], (unsigned long long)n_wanted);
-        if (n_fetched) atomicAdd(&c->evals[stripe], (unsigned long long)n_fetched);
+        if (n_fetched && !sketching) atomicAdd(&c->evals[stripe], (unsigned long long)n_fetched);
         if (n_sketched) atomicAdd(&c->sketched[stripe], (unsigned long long)n_sketched);
     }
     if (resample && lane == 0) {
@@ -908,9 +901,8 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
         atomicAdd(&probe_hits_s, n_wanted - n_fetched);
     }
     __syncthreads();
-    if (resample && tid == 0) s.memo_rate[row] = probe_asked_s > 0 ? (probe_hits_s * 256) / probe_asked_s : 256;
-    const KeptCount kept{resample ? s.memo_rate + row : nullptr, &c->sketch_rows, &probe_hits_s, &probe_asked_s,
-                         s.sketch_min_rate, a.m};
+    if (resample && tid == 0)
+        s.memo_rate[row] = (probe_asked_s > 0 ? (probe_hits_s * 256) / probe_asked_s : 256) | (memo_word & (1 << 16));
     // ---- merge: ann.py:75-88 ----
     if constexpr (SCPL > 0) {
         // A sketched row knows every candidate distance only as lo <= d <= hi (ld holds lo, le holds hi).
@@ -930,7 +922,7 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
             const float wv_d = nva > 0 ? vl_key_dist(wv) : -1.0f;
             for (int i = tid; i < a.m; i += THREADS) {
                 const int32_t cid = li[i];
-                uint8_t f = 0;
+                uint8_t f = flags[i] & 16;  // set by the expand phase for a distance that came from the cache
                 if (cid != VL_MAXINT) {
                     const float lo = ld[i];
                     bool need = !(lo > ws_d);
@@ -942,26 +934,27 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
                 }
                 flags[i] = f;
             }
-            // The Vt distinct candidates with the smallest upper bounds among those certainly above wv
+            // The Vt candidates of distinct ids with the smallest upper bounds among those certainly above wv
             // (bit 8), found one block-wide minimum at a time; fewer than Vt of them: every one may be taken.
+            // Every copy of a chosen id is marked - copies may carry different bounds (one fresh from the sketch,
+            // one decoded from the cache) and must not count twice.
             bool all_rest = false;
             if (!seen_full) {
-                uint64_t last = 0ull;
                 for (int r = 0; r < a.Vt; ++r) {
                     uint64_t mine = kPadKey;
                     for (int i = tid; i < a.m; i += THREADS) {
-                        if (!(flags[i] & 2)) continue;
+                        if ((flags[i] & (2 | 8)) != 2) continue;
                         const uint64_t k = vl_make_key(li[i], le[i]);
-                        if ((r == 0 || k > last) && k < mine) mine = k;
+                        if (k < mine) mine = k;
                     }
                     const uint64_t mn = block_min_key(mine, red, r);
                     if (mn == kPadKey) {
                         all_rest = true;
                         break;
                     }
-                    last = mn;
+                    const int32_t chosen = vl_key_id(mn);
                     for (int i = tid; i < a.m; i += THREADS)
-                        if ((flags[i] & 2) && vl_make_key(li[i], le[i]) == mn) flags[i] |= 8;
+                        if ((flags[i] & 2) && li[i] == chosen) flags[i] |= 8;
                 }
             }
             int n_exact = 0, n_real = 0;
@@ -971,11 +964,11 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
                 const bool has = slot < a.m;
                 const int32_t cid = has ? li[slot] : VL_MAXINT;
                 const uint8_t f = has ? flags[slot] : 0;
-                const bool ok = (f & (4 | 8)) || (all_rest && (f & 2));
+                const bool ok = ((f & (4 | 8)) || (all_rest && (f & 2))) && !(f & 16);
                 if (ok) flags[slot] = f | 16;  // its distance is exact from here on
                 n_exact += __popcll(__ballot(ok));
-                n_real += __popcll(__ballot(cid != VL_MAXINT));
-                wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0, nullptr, 0, false);
+                n_real += __popcll(__ballot(cid != VL_MAXINT && !(f & 16)));  // candidates known by bounds only
+                wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0, memo_row, s.memo_shift, false);
             }
             __syncthreads();
             // tv: the largest exact distance of those Vt candidates.  Vt distinct unvisited candidates above wv
@@ -1003,7 +996,7 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
                     ld[slot] = VL_MAXFLOAT;
                 }
                 n_exact += __popcll(__ballot(ok));
-                wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0, nullptr, 0, false);
+                wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0, memo_row, s.memo_shift, false);
             }
             if (s.count_evals && lane == 0 && n_exact)
                 atomicAdd(&c->evals[(int)((blockIdx.x * (THREADS / kWave) + wave) & (kBeamStripes - 1))],
@@ -1026,9 +1019,9 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
                 __syncthreads();
             }
         };
-        merge_row<THREADS, true>(a, smem, pre, refine, kept);
+        merge_row<THREADS, true>(a, smem, pre, refine);
     } else {
-        merge_row<THREADS, true>(a, smem, pre, NoRefine(), kept);
+        merge_row<THREADS, true>(a, smem, pre);
     }
 }
 
@@ -1301,23 +1294,6 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     step.sketch = (sketch && !step.l2 && aligned && use_fused && p->dim <= 2048) ? sketch : nullptr;
     step.sketch_row_bytes = sketch_row_bytes(p->dim);
     step.sketch_chunks = (int)sketch_data_chunks(p->dim);
-    // With a sketch the alternative to the cache is no longer the whole row.  Per candidate, in bytes: the cache
-    // costs a 64-byte probe, and row + id + a 64-byte store for every miss; the sketch costs its row + id, and an
-    // exact evaluation for about one candidate in ten.  Above the share of hits at which the two are equal (0.66
-    // for 768 columns) a row is better off with the cache.
-    int sketch_rate = 0;
-    if (step.sketch) {
-        static const int rate_env = [] {
-            const char *e = getenv("VL_BEAM_SKETCH_MIN_RATE");
-            return e ? atoi(e) : -1;
-        }();
-        const double row = 4.0 * p->dim + 76.0, sk = (double)step.sketch_row_bytes + 4.0 + 0.10 * (4.0 * p->dim + 12.0);
-        int r = (int)(256.0 * (1.0 - (sk - 64.0) / row));
-        r = r < 0 ? 0 : (r > 255 ? 255 : r);
-        sketch_rate = r > step.memo_min_rate ? r : step.memo_min_rate;
-        if (rate_env >= 0) sketch_rate = rate_env;
-    }
-    step.sketch_min_rate = sketch_rate;
     step.memo_shift = 32;
     if (step.memo) {
         int lg = 0;
@@ -1325,8 +1301,8 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
         VL_REQUIRE((1 << lg) == l.memo_slots, "memo slots must be a power of two");
         step.memo_shift = 32 - lg;
     }
-    // every row starts with the sketch when there is one and no cache to prefer
-    const bool sketch_from_start = step.sketch && !step.memo;
+    // with a sketch every row starts out using it (and the cache, when there is one)
+    const bool sketch_from_start = step.sketch != nullptr;
     {
         int64_t n = p->n_rows * l.VL;
         if (n < kBeamStripes) n = kBeamStripes;
@@ -1375,11 +1351,9 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     // queue changes and the next check ends the loop.  More iterations than that mean the
     // control block was overwritten while the loop ran (a workspace shared by two calls).
     const int64_t t_limit = l.E + l.VL + 2 * (int64_t)R + 2;
-    // The kernel that can read the sketch holds more registers, so fewer rows are resident per compute unit, and
-    // one launch serves the whole batch: it takes over only when most rows of the batch would rather use the
-    // sketch than the cache.  Rows find that out in iteration kMemoDecide and are counted on the device; the
-    // host reads the count at its next progress check.  In the other kernel a row that prefers the sketch goes
-    // on as it would without one.  Without a cache every row uses the sketch from the start.
+    // One launch serves the whole batch: the kernel that can read the sketch is launched while most rows of the
+    // batch still use it.  A row gives the sketch up when it does not pay (counted on the device, read by the
+    // host at its regular progress check); in the other kernel such a row goes on as it would without a sketch.
     const uint8_t *sketch_table = step.sketch;
     int sketch_rows = sketch_from_start ? (int)p->n_rows : 0;
     int64_t t = 0;
@@ -1414,7 +1388,7 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
         }
         int changed = 0;
         VL_HIP(hipMemcpyAsync(&changed, &ctrl->changed[(t / R) & 63], sizeof(int), hipMemcpyDeviceToHost, st));
-        if (sketch_table && t >= kMemoDecide)
+        if (sketch_table)
             VL_HIP(hipMemcpyAsync(&sketch_rows, &ctrl->sketch_rows, sizeof(int), hipMemcpyDeviceToHost, st));
         VL_HIP(hipStreamSynchronize(st));
         if (prof) {

@@ -30,6 +30,21 @@ __device__ __forceinline__ void memo_store(uint64_t *memo_row, int shift, int32_
 __device__ __forceinline__ uint64_t memo_load(const uint64_t *memo_row, int shift, int32_t id) {
     return __hip_atomic_load(memo_row + memo_hash(id, shift), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// A second kind of entry, for rows that know a candidate only through the 8-bit sketch (cosine distances,
+// which lie in [0, 1]): bit 31 of the id word set (ids stay below 2^30), and in place of the distance its
+// bounds lo <= d <= hi as 16-bit fixed point, each moved one step outwards so that encoding and decoding
+// never narrow them.
+constexpr uint32_t kMemoBounds = 0x80000000u;
+__device__ __forceinline__ void memo_store_bounds(uint64_t *memo_row, int shift, int32_t id, float lo, float hi) {
+    int l = lo >= 0.0f ? (int)(lo * 65535.0f) - 1 : 0;   // a NaN bound becomes the widest one
+    int h = hi <= 1.0f ? (int)(hi * 65535.0f) + 2 : 65535;
+    l = l < 0 ? 0 : l;
+    h = h > 65535 ? 65535 : h;
+    uint64_t e = ((uint64_t)(((uint32_t)l << 16) | (uint32_t)h) << 32) | ((uint32_t)id | kMemoBounds);
+    __hip_atomic_store(memo_row + memo_hash(id, shift), e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float memo_bound_lo(uint64_t e) { return (float)(uint32_t)(e >> 48) * (1.0f / 65535.0f); }
+__device__ __forceinline__ float memo_bound_hi(uint64_t e) { return (float)((uint32_t)(e >> 32) & 0xffffu) * (1.0f / 65535.0f); }
 
 // Folds the partial sums of a group of LPR lanes: lane l += lane l + h for h = LPR/2 ... 1, so the
 // group's first lane ends with the sum in the fixed order.  Steps of 32 and 16 lanes swap register

@@ -105,7 +105,8 @@ __device__ __forceinline__ void sketch_query_load(SketchQuery<SCPL> &sq, const f
 template <int SCPL, int SLPR, int SU>
 __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const uint8_t *__restrict__ table,
                                             int64_t row_bytes, int data_chunks, int32_t my_id, bool ok,
-                                            float *__restrict__ out_lo, float *__restrict__ out_hi) {
+                                            float *__restrict__ out_lo, float *__restrict__ out_hi,
+                                            uint64_t *memo_row = nullptr, int memo_shift = 0) {
     constexpr int G = kWave / SLPR;
     const int lane = threadIdx.x & (kWave - 1);
     const int grp = lane / SLPR;
@@ -113,6 +114,7 @@ __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const u
     uint64_t mask = __ballot(ok);
     while (mask) {
         int mysrc[SU];
+        int32_t ids[SU];
         uint4 r[SU][SCPL];
         float4 tail[SU];
 #pragma unroll
@@ -129,6 +131,7 @@ __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const u
             }
             mysrc[u] = s;
             const int32_t id = __shfl(my_id, s >= 0 ? s : 0);
+            ids[u] = id;
             const uint4 *row = reinterpret_cast<const uint4 *>(table + (int64_t)id * row_bytes);
 #pragma unroll
             for (int i = 0; i < SCPL; ++i) {
@@ -160,8 +163,10 @@ __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const u
                 // multiply-add per lane, up to six adds across lanes, two products) each round by 2^-24 of at most
                 // ||q^|| ||v^||
                 const float eps = (sq.norm2 * resid + (sq.qerr + 4e-6f * sq.norm2) * (norm + resid) + sq.exactc * norm) * 1.0001f + 2e-7f;
-                out_lo[mysrc[u]] = clamp_distance(s_hat + eps);
-                out_hi[mysrc[u]] = clamp_distance(s_hat - eps);
+                const float lo = clamp_distance(s_hat + eps), hi = clamp_distance(s_hat - eps);
+                out_lo[mysrc[u]] = lo;
+                out_hi[mysrc[u]] = hi;
+                if (memo_row) memo_store_bounds(memo_row, memo_shift, ids[u], lo, hi);
             }
         }
     }
