@@ -1001,17 +1001,18 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
             if (s.count_evals && lane == 0 && n_exact)
                 atomicAdd(&c->evals[(int)((blockIdx.x * (THREADS / kWave) + wave) & (kBeamStripes - 1))],
                           (unsigned long long)n_exact);
-            // A row that has to evaluate more than half of its candidates exactly after all (its candidates lie
-            // within the sketch's error of the queues' last slots: real neighbour lists) gives the sketch up for
-            // the rest of the call.  Not before iteration kMemoDecide: the first iterations fill the visit queue
-            // and keep everything.
-            if (t > kMemoDecide) {
+            // A row that has to evaluate more than half of the candidates it knew by bounds exactly after all
+            // (they lie within the sketch's error of the queues' last slots: real neighbour lists) gives the
+            // sketch up for the rest of the call.  The first iterations fill the visit queue and keep a lot, so
+            // until iteration kMemoDecide only a row that evaluates nearly all of them (7 in 8) does.
+            if (t > 2 && !resample) {  // (the iteration that measures the cache uses the same two counters)
                 if (lane == 0) {
                     atomicAdd(&probe_asked_s, n_real);
                     atomicAdd(&probe_hits_s, n_exact);
                 }
                 __syncthreads();
-                if (tid == 0 && 2 * probe_hits_s > probe_asked_s) {
+                const bool quit = t > kMemoDecide ? 2 * probe_hits_s > probe_asked_s : 8 * probe_hits_s > 7 * probe_asked_s;
+                if (tid == 0 && quit) {
                     s.memo_rate[row] = memo_rate;
                     atomicAdd(&c->sketch_rows, -1);
                 }
