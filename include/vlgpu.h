@@ -252,8 +252,10 @@ int vl_sketch_build(const float *vectors, int64_t n_vectors, int64_t dim,
 /* vl_closest_vectors with the sketch of `vectors` (NULL: exactly
  * vl_closest_vectors).  Same arguments, same result, same return value.  The
  * sketch serves the fused step under the cosine metric for 16-byte aligned rows
- * of up to 2048 columns; other calls ignore it.  Each row decides for itself:
- * rows whose candidates mostly repeat keep the distance cache instead. */
+ * of up to 2048 columns; other calls ignore it.  The distance cache then also
+ * remembers candidates that were only bounded, so a repeat costs neither a
+ * sketch row nor a vector row.  A row whose bounded candidates mostly need
+ * their exact distance after all gives the sketch up for the rest of the call. */
 int64_t vl_closest_vectors_with_sketch(const vl_beam_params *p,
                                        const float *queries, const float *vectors,
                                        const uint8_t *sketch,

@@ -669,7 +669,7 @@ struct StepArgs {
     uint32_t width_magic;  // floor(2^32 / width) + 1: slot / width == umulhi(slot, width_magic) for slot * width < 2^32
     uint64_t *memo;
     int memo_shift;
-    int32_t *memo_rate;   // per row: share (x 256) of the candidates of iteration kMemoDecide that were cached; bit 16: the row prefers the sketch
+    int32_t *memo_rate;   // per row: share (x 256) of the candidates of iteration kMemoDecide that were cached; bit 16: the row uses the sketch
     int memo_min_rate;    // the cache stays in use only if that share is at least this (x 256)
     int count_evals;
     int l2;  // 0: cosine distance, 1: squared L2
@@ -693,10 +693,10 @@ constexpr int kMemoDecide = 9;
 constexpr int kPreQ = 2, kPreV = 2, kPreS = 4;
 
 // SCPL > 0: the kernel can look at candidates through the sketch first (SCPL chunks per lane, SLPR lanes
-// per sketch row, SU loads in flight).  A row does so once it has left the distance cache alone (a cache
-// hit is cheaper still, so rows whose candidates repeat keep the cache instead): it gets bounds for all
-// candidates from a quarter of the bytes, then exact distances for the few whose lower bound is not above
-// every threshold that decides what the merge phase keeps.
+// per sketch row, SU loads in flight).  A row that does so gets bounds for the candidates the distance cache
+// does not know from a quarter of the bytes, then exact distances for the few whose lower bound is not above
+// every threshold that decides what the merge phase keeps; it stops doing so when most of them turn out to
+// need their exact distance (bit 16 of its word in memo_rate: set at the start of the call, cleared then).
 template <int CPL, int LPR, int U, bool GENERIC, int THREADS, int SCPL = 0, int SLPR = 64, int SU = 1>
 __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
     extern __shared__ __align__(16) unsigned char smem[];
