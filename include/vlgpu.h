@@ -206,6 +206,10 @@ typedef struct vl_beam_params {
  * (id, distance) pairs: the workspace shrinks by the cache's table and every
  * candidate distance is evaluated when it is asked for. */
 #define VL_BEAM_NO_CACHE 8
+/* The call brings the 8-bit sketch of the vector table
+ * (vl_closest_vectors_with_sketch): the workspace then also holds the call's
+ * query rows rounded for it (32 bytes per 16 columns and row). */
+#define VL_BEAM_USES_SKETCH 16
 
 int64_t vl_beam_workspace_bytes(const vl_beam_params *p);
 
@@ -255,7 +259,9 @@ int vl_sketch_build(const float *vectors, int64_t n_vectors, int64_t dim,
  * of up to 2048 columns; other calls ignore it.  The distance cache then also
  * remembers candidates that were only bounded, so a repeat costs neither a
  * sketch row nor a vector row.  A row whose bounded candidates mostly need
- * their exact distance after all gives the sketch up for the rest of the call. */
+ * their exact distance after all gives the sketch up for the rest of the call.
+ * p->flags must hold VL_BEAM_USES_SKETCH, also in the vl_beam_workspace_bytes
+ * call that sized the workspace. */
 int64_t vl_closest_vectors_with_sketch(const vl_beam_params *p,
                                        const float *queries, const float *vectors,
                                        const uint8_t *sketch,

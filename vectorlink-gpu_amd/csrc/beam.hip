@@ -31,6 +31,8 @@ int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors,
                      int seen_cols, int64_t visit_stride, int count_evals, uint64_t *memo, int memo_slots,
                      int metric, hipStream_t st);
 
+int vl_launch_sketch_queries(const float *queries, int64_t n_rows, int64_t dim, uint8_t *out_rows, hipStream_t st);
+
 namespace {
 
 constexpr int kMaxVisit = 64;  // parallel_visit_count handled by one wavefront
@@ -676,6 +678,8 @@ struct StepArgs {
     const uint8_t *sketch;     // 8-bit sketch of `vectors` (sketch_device.h), or null
     int64_t sketch_row_bytes;
     int sketch_chunks;         // 16-byte chunks of data in a sketch row
+    const uint8_t *rounded_queries;  // the call's query rows rounded for the sketch (sketch_device.h)
+    int64_t rounded_query_bytes;
 };
 
 // A probe of the distance cache is a random 8-byte read and every evaluated distance a random 8-byte
@@ -830,7 +834,7 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
     if constexpr (SCPL > 0) {
         if (sketching) {
             SketchQuery<SCPL> sq;
-            sketch_query_load<SCPL, SLPR>(sq, q_row, s.dim);
+            sketch_query_load<SCPL, SLPR>(sq, s.rounded_queries + row * s.rounded_query_bytes, s.sketch_chunks);
             for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
                 if (c0 != wave * kWave) id = resolve(c0);
                 const int slot = c0 + lane;
@@ -1104,7 +1108,7 @@ int launch_step_by_dim(const StepArgs &s, bool aligned, int threads, size_t smem
 
 struct BeamLayout {
     int64_t m, VL, Vt, E, head;
-    int64_t off_cand_ids, off_cand_d, off_v_ids, off_v_d, off_seen, off_seen_count, off_row_quiet, off_memo_rate, off_ctrl, off_memo, total;
+    int64_t off_cand_ids, off_cand_d, off_v_ids, off_v_d, off_seen, off_seen_count, off_row_quiet, off_memo_rate, off_ctrl, off_rounded, off_memo, total;
     int memo_slots;
 };
 
@@ -1145,6 +1149,8 @@ int beam_layout(const vl_beam_params *p, BeamLayout *l, bool lean = false) {
     l->off_row_quiet = o; o = align256(o + p->n_rows * 4);
     l->off_memo_rate = o; o = align256(o + p->n_rows * 4);
     l->off_ctrl = o; o = align256(o + (int64_t)sizeof(BeamCtrl));
+    // the query rows rounded for the sketch, for calls that say they bring one
+    l->off_rounded = o; o = align256(o + ((p->flags & VL_BEAM_USES_SKETCH) && !lean ? p->n_rows * sketch_query_bytes(p->dim) : 0));
     // per-row cache of evaluated (id, distance) pairs: 128 slots per candidate of one iteration,
     // 1Ki..64Ki per row, the whole table at most 8 GiB (measured at 1M x 768: 16Ki -> 64Ki slots cuts the
     // rows fetched in the second optimisation loop by 30 %, 256Ki adds little)
@@ -1293,6 +1299,10 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     }
     // The sketch serves the cosine distance of 16-byte aligned rows in the fused step; other calls ignore it.
     step.sketch = (sketch && !step.l2 && aligned && use_fused && p->dim <= 2048) ? sketch : nullptr;
+    VL_REQUIRE(!step.sketch || (p->flags & VL_BEAM_USES_SKETCH),
+               "a call with a sketch needs VL_BEAM_USES_SKETCH in flags (and a workspace sized with it)");
+    step.rounded_queries = (const uint8_t *)(ws + l.off_rounded);
+    step.rounded_query_bytes = sketch_query_bytes(p->dim);
     step.sketch_row_bytes = sketch_row_bytes(p->dim);
     step.sketch_chunks = (int)sketch_data_chunks(p->dim);
     step.memo_shift = 32;
@@ -1304,6 +1314,10 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     }
     // with a sketch every row starts out using it (and the cache, when there is one)
     const bool sketch_from_start = step.sketch != nullptr;
+    if (step.sketch) {
+        rc = vl_launch_sketch_queries(queries, p->n_rows, p->dim, (uint8_t *)(ws + l.off_rounded), st);
+        if (rc < 0) return rc;
+    }
     {
         int64_t n = p->n_rows * l.VL;
         if (n < kBeamStripes) n = kBeamStripes;

@@ -71,7 +71,69 @@ __global__ __launch_bounds__(256) void sketch_build_kernel(const float *__restri
     }
 }
 
+// Rounds the query rows of a call to 15 bits per element for the sketch (sketch_device.h): one wavefront per
+// row, a lane rounds four elements at a time.
+__global__ __launch_bounds__(256) void sketch_query_kernel(const float *__restrict__ queries, int64_t n, int dim,
+                                                           int64_t row0, uint8_t *__restrict__ out_rows) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t row = row0 + (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+    if (row >= n) return;
+    const float *q = queries + row * dim;
+    const int chunks = (int)sketch_data_chunks(dim);
+    uint8_t *out = out_rows + row * sketch_query_bytes(dim);
+    float mx = 0.f, n2 = 0.f;
+    for (int j = lane; j < dim; j += kWave) {
+        const float x = q[j];
+        mx = fmaxf(mx, __builtin_fabsf(x));   // a NaN is not seen here but makes n2 a NaN
+        n2 = __builtin_fmaf(x, x, n2);
+    }
+    mx = wave_max(mx);
+    n2 = wave_sum(n2);
+    // a row of zeros, of denormals, or one with a NaN: rounded to zero, and the bound is the row's whole length
+    const bool tiny = !(mx > 1e-30f) || !(n2 == n2);
+    const float inv = tiny ? 0.f : 16256.0f / mx;
+    for (int g = lane; g < chunks * 4; g += kWave) {   // word g of the row: elements 4g .. 4g + 3
+        uint32_t hi = 0, lo = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int j = 4 * g + k;
+            int v = 0;
+            if (j < dim) v = (int)fminf(fmaxf(rintf(q[j] * inv), -16256.0f), 16256.0f);
+            const int l = ((v + 64) & 127) - 64;   // [-64, 63]
+            const int h = (v - l) >> 7;            // [-127, 127], v = 128 h + l
+            hi |= (uint32_t)(h & 0xff) << (8 * k);
+            lo |= (uint32_t)(l & 0xff) << (8 * k);
+        }
+        const int c = g >> 2, w = g & 3;
+        reinterpret_cast<uint32_t *>(out)[c * 8 + w] = hi;
+        reinterpret_cast<uint32_t *>(out)[c * 8 + 4 + w] = lo;
+    }
+    if (lane == 0) {
+        float4 tail;
+        tail.x = mx / 16256.0f;
+        tail.y = __builtin_sqrtf(n2) * 1.001f;
+        // an element moves by at most half a step (0.51: q * inv and the step itself are rounded floats); a NaN or
+        // an infinity in the query makes the bound a NaN or an infinity, which the callers read as "evaluate"
+        tail.z = tiny ? tail.y : 0.51f * tail.x * __builtin_sqrtf((float)(16 * chunks));
+        tail.w = (float)(dim + 16) * 5.9604645e-8f * tail.y;  // terms |q_j v_j| sum to at most ||q||_2 ||v||_2
+        *reinterpret_cast<float4 *>(out + (int64_t)chunks * 32) = tail;
+    }
+}
+
 }  // namespace
+
+// Rounded query rows for a beam-search call that uses the sketch; out_rows: n_rows x sketch_query_bytes(dim),
+// 16-byte aligned (part of the call's workspace).
+int vl_launch_sketch_queries(const float *queries, int64_t n_rows, int64_t dim, uint8_t *out_rows, hipStream_t st) {
+    const int rows_per_block = 256 / kWave;
+    for (int64_t row0 = 0; row0 < n_rows; row0 += kMaxBlocks * rows_per_block) {
+        int64_t rows = n_rows - row0 < kMaxBlocks * rows_per_block ? n_rows - row0 : kMaxBlocks * rows_per_block;
+        hipLaunchKernelGGL(sketch_query_kernel, dim3((unsigned)((rows + rows_per_block - 1) / rows_per_block)), dim3(256),
+                           0, st, queries, n_rows, (int)dim, row0, out_rows);
+        VL_LAUNCH_CHECK("sketch_query_kernel");
+    }
+    return VL_OK;
+}
 
 VL_EXPORT int64_t vl_sketch_row_bytes(int64_t dim) {
     if (dim <= 0) {

@@ -51,52 +51,32 @@ struct SketchQuery {
     float exactc;  // per unit of ||v||_2: bound on the rounding of the exact kernel's dot product
 };
 
+// The rounded query rows of a call are made once, by sketch_query_kernel (sketch.hip), and kept in the call's
+// workspace: per row and 16-element chunk 16 high digits then 16 low digits (int8), and after the last chunk
+// float qscale, norm2, qerr, exactc.
+__host__ __device__ inline int64_t sketch_query_bytes(int64_t dim) { return sketch_data_chunks(dim) * 32 + 16; }
+
 template <int SCPL, int SLPR>
-__device__ __forceinline__ void sketch_query_load(SketchQuery<SCPL> &sq, const float *__restrict__ q_row, int dim) {
+__device__ __forceinline__ void sketch_query_load(SketchQuery<SCPL> &sq, const uint8_t *__restrict__ rounded_row,
+                                                  int data_chunks) {
     const int lig = (threadIdx.x & (kWave - 1)) % SLPR;
-    float4 x[SCPL][4];
-    float mx = 0.f, n = 0.f;
+    const uint4 *words = reinterpret_cast<const uint4 *>(rounded_row);
 #pragma unroll
     for (int i = 0; i < SCPL; ++i) {
         const int c = lig + SLPR * i;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const int j = 16 * c + 4 * w;  // dim is a multiple of 4 on this path
-            x[i][w] = j < dim ? *reinterpret_cast<const float4 *>(q_row + j) : make_float4(0.f, 0.f, 0.f, 0.f);
-            mx = fmaxf(fmaxf(mx, fmaxf(__builtin_fabsf(x[i][w].x), __builtin_fabsf(x[i][w].y))),
-                       fmaxf(__builtin_fabsf(x[i][w].z), __builtin_fabsf(x[i][w].w)));
-            n = __builtin_fmaf(x[i][w].x, x[i][w].x, n); n = __builtin_fmaf(x[i][w].y, x[i][w].y, n);
-            n = __builtin_fmaf(x[i][w].z, x[i][w].z, n); n = __builtin_fmaf(x[i][w].w, x[i][w].w, n);
+        uint4 h = make_uint4(0u, 0u, 0u, 0u), l = h;
+        if (c < data_chunks) {
+            h = words[2 * c];
+            l = words[2 * c + 1];
         }
+        sq.qh[i][0] = (int)h.x; sq.qh[i][1] = (int)h.y; sq.qh[i][2] = (int)h.z; sq.qh[i][3] = (int)h.w;
+        sq.ql[i][0] = (int)l.x; sq.ql[i][1] = (int)l.y; sq.ql[i][2] = (int)l.z; sq.ql[i][3] = (int)l.w;
     }
-#pragma unroll
-    for (int h = SLPR / 2; h >= 1; h >>= 1) {  // every lane of the group ends with the totals
-        mx = fmaxf(mx, __shfl_xor(mx, h));
-        n += __shfl_xor(n, h);
-    }
-    // a row of zeros, of denormals, or one with a NaN: rounded to zero, and the bound is the row's whole length
-    const bool tiny = !(mx > 1e-30f);
-    const float inv = tiny ? 0.f : 16256.0f / mx;
-    auto digits = [&](float v, int &hi, int &lo) {
-        const int q = (int)fminf(fmaxf(rintf(v * inv), -16256.0f), 16256.0f);
-        lo = ((q + 64) & 127) - 64;   // [-64, 63]
-        hi = (q - lo) >> 7;           // [-127, 127], q = 128 hi + lo
-    };
-#pragma unroll
-    for (int i = 0; i < SCPL; ++i)
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            int h0, l0, h1, l1, h2, l2, h3, l3;
-            digits(x[i][w].x, h0, l0); digits(x[i][w].y, h1, l1); digits(x[i][w].z, h2, l2); digits(x[i][w].w, h3, l3);
-            sq.qh[i][w] = (h0 & 0xff) | ((h1 & 0xff) << 8) | ((h2 & 0xff) << 16) | ((h3 & 0xff) << 24);
-            sq.ql[i][w] = (l0 & 0xff) | ((l1 & 0xff) << 8) | ((l2 & 0xff) << 16) | ((l3 & 0xff) << 24);
-        }
-    sq.qscale = mx / 16256.0f;
-    sq.norm2 = __builtin_sqrtf(n) * 1.001f;
-    // an element moves by at most half a step (0.51: v * inv and the step itself are rounded floats); a NaN or an
-    // infinity in the query makes the bound a NaN or an infinity, which the callers read as "evaluate"
-    sq.qerr = tiny ? sq.norm2 : 0.51f * sq.qscale * __builtin_sqrtf((float)(16 * SCPL * SLPR));
-    sq.exactc = (float)(dim + 16) * 5.9604645e-8f * sq.norm2;  // terms |q_j v_j| sum to at most ||q||_2 ||v||_2
+    const float4 tail = *reinterpret_cast<const float4 *>(rounded_row + (int64_t)data_chunks * 32);
+    sq.qscale = tail.x;
+    sq.norm2 = tail.y;
+    sq.qerr = tail.z;
+    sq.exactc = tail.w;
 }
 
 // One wavefront: lane j holds candidate id `my_id` (valid when `ok`); the bounds of its distance to

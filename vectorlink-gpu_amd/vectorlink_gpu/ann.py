@@ -27,6 +27,7 @@ BEAM_TWO_LAUNCHES = 1  # include/vlgpu.h: VL_BEAM_TWO_LAUNCHES
 BEAM_SORT_MERGE = 2    # include/vlgpu.h: VL_BEAM_SORT_MERGE
 BEAM_PER_QUERY_STOP = 4  # include/vlgpu.h: VL_BEAM_PER_QUERY_STOP (a different loop: every row stops on its own)
 BEAM_NO_CACHE = 8  # include/vlgpu.h: VL_BEAM_NO_CACHE (no per-row cache of evaluated distances; same result)
+BEAM_USES_SKETCH = 16  # include/vlgpu.h: VL_BEAM_USES_SKETCH (set by closest_vectors when it is given a sketch)
 
 
 def _beam_params(batch: int, dim: int, n_vectors: int, width: int, queue: Queue, config: Dict,
@@ -163,7 +164,7 @@ def closest_vectors(query_vecs: Tensor, search_queue: Queue, vectors: Tensor, be
         assert exclude.dtype == torch.int32 and exclude.size(0) == batch
         excl = exclude.contiguous()
     p = _beam_params(batch, dim, vectors.size(0), beams.size(1), search_queue, config,
-                     0 if excl is None else excl.size(1), flags)
+                     0 if excl is None else excl.size(1), flags | (BEAM_USES_SKETCH if sketch is not None else 0))
     need = nv.check(nv.lib().vl_beam_workspace_bytes(ctypes.byref(p)))
     workspace = _workspace(vectors.device)
     with workspace.lock:
