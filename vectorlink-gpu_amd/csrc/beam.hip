@@ -1046,7 +1046,7 @@ void beam_step_sketch_kernel(StepArgs s) {
     beam_step_body<CPL, LPR, U, false, THREADS, SCPL, SLPR, SU>(s);
 }
 
-template <int CPL, int LPR, int U, bool GENERIC, int SCPL = 0, int SLPR = 64, int SU = 1, int WPE = 4>
+template <int CPL, int LPR, int U, bool GENERIC, int SCPL = 0, int SLPR = 64, int SU = 1, int WPE = 4, int UX = U>
 void launch_step(const StepArgs &s, int threads, size_t smem, hipStream_t st) {
     dim3 grid((unsigned)s.m.n_rows);
     if constexpr (SCPL > 0) {
@@ -1054,11 +1054,11 @@ void launch_step(const StepArgs &s, int threads, size_t smem, hipStream_t st) {
     }
     if constexpr (SCPL > 0) {
         if (threads == 128) {
-            auto kernel = beam_step_sketch_kernel<CPL, LPR, U, 128, SCPL, SLPR, SU, WPE>;
+            auto kernel = beam_step_sketch_kernel<CPL, LPR, UX, 128, SCPL, SLPR, SU, WPE>;
             if (vl_allow_lds(kernel, smem) != hipSuccess) return;  // seen by the launch check
             hipLaunchKernelGGL(kernel, grid, dim3(128), smem, st, s);
         } else {
-            auto kernel = beam_step_sketch_kernel<CPL, LPR, U, 256, SCPL, SLPR, SU, WPE>;
+            auto kernel = beam_step_sketch_kernel<CPL, LPR, UX, 256, SCPL, SLPR, SU, WPE>;
             if (vl_allow_lds(kernel, smem) != hipSuccess) return;
             hipLaunchKernelGGL(kernel, grid, dim3(256), smem, st, s);
         }
@@ -1084,8 +1084,10 @@ int dist_variant() {
 }
 
 // The numbers after `false` are the sketch's lane shape for rows of that size (chunks per lane, lanes per row,
-// loads in flight) and the wavefronts per SIMD asked for: a sketch row has a quarter of the chunks, so a quarter
-// of the lanes (or of the chunks per lane) covers it.
+// loads in flight), the wavefronts per SIMD asked for and, where given, the whole rows in flight in the sketch
+// kernel (it fetches few of them, so fewer in flight cost nothing and leave registers for another wavefront:
+// 0.40 -> 0.36 ms per launch at 384 columns): a sketch row has a quarter of the chunks, so a quarter of the
+// lanes (or of the chunks per lane) covers it.
 int launch_step_by_dim(const StepArgs &s, bool aligned, int threads, size_t smem, hipStream_t st) {
     const int nchunks = s.nchunks;
     const int variant = dist_variant();
@@ -1094,14 +1096,14 @@ int launch_step_by_dim(const StepArgs &s, bool aligned, int threads, size_t smem
     else if (nchunks <= 32 && variant == 1) launch_step<1, 32, 8, false>(s, threads, smem, st);
     else if (nchunks <= 32) launch_step<2, 16, 4, false, 1, 8, 4, 5>(s, threads, smem, st);
     else if (nchunks <= 64) launch_step<1, 64, 8, false, 2, 8, 2, 5>(s, threads, smem, st);
-    else if (nchunks <= 96 && variant != 1) launch_step<3, 32, 4, false, 3, 8, 2, 5>(s, threads, smem, st);
-    else if (nchunks <= 128) launch_step<2, 64, 8, false, 2, 16, 2, 5>(s, threads, smem, st);
+    else if (nchunks <= 96 && variant != 1) launch_step<3, 32, 4, false, 3, 8, 2, 6, 2>(s, threads, smem, st);
+    else if (nchunks <= 128) launch_step<2, 64, 8, false, 2, 16, 2, 6, 2>(s, threads, smem, st);
     else if (nchunks <= 192) launch_step<3, 64, 4, false, 3, 16, 2, 5>(s, threads, smem, st);
-    else if (nchunks <= 256) launch_step<4, 64, 4, false, 4, 16, 2, 4>(s, threads, smem, st);
-    else if (nchunks <= 320) launch_step<5, 64, 2, false, 3, 32, 2, 5>(s, threads, smem, st);
-    else if (nchunks <= 384) launch_step<6, 64, 2, false, 3, 32, 2, 5>(s, threads, smem, st);
-    else if (nchunks <= 448) launch_step<7, 64, 2, false, 4, 32, 2, 4>(s, threads, smem, st);
-    else launch_step<8, 64, 2, false, 4, 32, 2, 4>(s, threads, smem, st);
+    else if (nchunks <= 256) launch_step<4, 64, 4, false, 4, 16, 2, 5, 2>(s, threads, smem, st);
+    else if (nchunks <= 320) launch_step<5, 64, 2, false, 3, 32, 2, 6, 1>(s, threads, smem, st);
+    else if (nchunks <= 384) launch_step<6, 64, 2, false, 3, 32, 2, 6, 1>(s, threads, smem, st);
+    else if (nchunks <= 448) launch_step<7, 64, 2, false, 4, 32, 2, 5, 1>(s, threads, smem, st);
+    else launch_step<8, 64, 2, false, 4, 32, 2, 5, 1>(s, threads, smem, st);
     VL_LAUNCH_CHECK("beam_step_kernel");
     return VL_OK;
 }
