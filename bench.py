@@ -46,7 +46,7 @@ MFMA_FP32_PEAK = 157.3  # MI355X published dense fp32 matrix TFLOP/s
 # (FETCH_SIZE x 2.0 after calibration against the 1 GiB copy + WRITE_SIZE x 1.0, "roofline pass" phases);
 # NOT measured in this run.  Workloads without a recorded counter run report null.
 TRAFFIC_PER_LOOP = {
-    "mix-1m-768": [(2540165.5 * 2 + 42010.7) * 1024, (823540.8 * 2 + 61712.4) * 1024, (573028.6 * 2 + 32363.5) * 1024],
+    "mix-1m-768": [(2543168.7 * 2 + 42128.0) * 1024, (821963.7 * 2 + 61734.6) * 1024, (578636.6 * 2 + 32422.2) * 1024],
     "mix-1m-128": [(436666.3 * 2 + 25910.0) * 1024, (231534.4 * 2 + 28947.1) * 1024, (153222.4 * 2 + 20410.1) * 1024],
 }
 
