@@ -773,7 +773,9 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
     const bool resample = memo_row && t == kMemoDecide;
     if (memo_row && memo_rate < s.memo_min_rate) memo_row = nullptr;
     bool sketching = false;
-    if constexpr (SCPL > 0) sketching = (memo_word >> 16) != 0;
+    // (not in the first iteration: the visit queue starts with empty slots, so everything unvisited is kept and
+    // would be fetched anyway)
+    if constexpr (SCPL > 0) sketching = (memo_word >> 16) != 0 && t > 1;
     const bool probing = memo_row != nullptr;
     if (tid < a.Vt) g_visit_s[tid] = my_visit;
     if (tid == 0) {
@@ -1381,7 +1383,7 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
             a.iter = (int)t;
             if (use_fused) {
                 step.m = a;
-                step.sketch = 2 * (int64_t)sketch_rows >= p->n_rows ? sketch_table : nullptr;
+                step.sketch = (t > 1 && 2 * (int64_t)sketch_rows >= p->n_rows) ? sketch_table : nullptr;
                 rc = launch_step_by_dim(step, aligned, merge_threads == 128 ? 128 : 256, smem, st);
                 if (rc < 0) return rc;
                 if (prof) VL_HIP(hipEventRecord(ev[3 * r + 1], st));
