@@ -326,3 +326,53 @@ def test_tables_with_more_rows_than_one_launch_holds():
     clear = (best.values[:, 1] - best.values[:, 0]) > 1e-5
     assert torch.equal(ki[tail][clear, 0].long(), best.indices[clear, 0])
     assert bool((ki[:300, 0] == torch.arange(300, device=DEV)).all())
+
+
+@pytest.mark.parametrize("workload,n", [("mix-1m-768", 300_000), ("zipf-20m-384", 400_000), ("mix-10m-1536", 150_000)])
+def test_sketch_and_plain_paths_agree_at_scale(workload, n):
+    """Two independent code paths over the same inputs at the benchmark row sizes: batches of 10,000 rows against
+    the circulant graph and against the graph one optimisation loop leaves, searched (a) as before the sketch
+    existed, (b) through the sketch alone, (c) with cache and sketch together.  Same iteration count, ids and
+    distance bits; the counters show that (b) and (c) did fetch fewer rows."""
+    say(f"sketch and plain paths, {workload} cut to {n}")
+    import ctypes
+
+    from vectorlink_gpu import Queue, synthetic
+    from vectorlink_gpu import _native as nv
+    from vectorlink_gpu.ann import BEAM_NO_CACHE, GraphBuild, closest_vectors, excluding_self
+    from vectorlink_gpu.kernels import build_sketch
+
+    base, _, w = synthetic.make(workload, n=n)
+    kw = synthetic.ann_kwargs(w)
+    c = dict(orc.DEFAULT_CONFIG)
+    c.update(kw)
+    c.update(optimization_loops=1, batch_size=10_000)
+    v = base.to(DEV)
+    build = GraphBuild(v, c, keep_history=True)
+    for _ in build.steps():
+        pass
+    ql = c["beam_size"] * c["beam_queue_factor"]
+    sk = build_sketch(v)
+    rows = 10_000
+    for state, (tb, td) in enumerate([build.history[0], (build.beams, build.distances)]):
+        results = []
+        for name, flags, sketch in (("plain", 0, None), ("sketch", BEAM_NO_CACHE, sk), ("cache+sketch", 0, sk)):
+            q = Queue(rows, ql, ql + ql * c["parallel_visit_count"], device=DEV)
+            q.insert(tb[n - rows:], td[n - rows:])
+            out = (ctypes.c_double * 9)()
+            nv.lib().vl_beam_profile(1, 1, out)
+            try:
+                t = closest_vectors(v[n - rows:], q, v, tb, c, excluding_self(n - rows, n, device=DEV), flags=flags,
+                                    sketch=sketch)
+            finally:
+                nv.lib().vl_beam_profile(0, 1, out)
+            say(f"  state {state} {name}: {t} iterations, rows fetched {out[4]:.0f}, through the sketch {out[8]:.0f}")
+            results.append((t, q.indices[:, :ql].clone(), q.distances[:, :ql].clone(), out[4], out[8]))
+        (t0, i0, d0, fetched0, _) = results[0]
+        for (t, i, d, fetched, sketched) in results[1:]:
+            assert t == t0
+            assert torch.equal(i, i0)
+            assert torch.equal(d.view(torch.int32), d0.view(torch.int32))
+            assert sketched > 0
+        if state == 0:
+            assert results[1][3] < 0.5 * fetched0 and results[2][3] < 0.5 * fetched0
