@@ -264,8 +264,10 @@ class GraphBuild:
                     queue.insert(self.beams.narrow(0, start, end - start), seed_distances.narrow(0, start, end - start))
                     if self.sketch is not None:
                         # the neighbour lists of a circulant graph share little, so a search of it meets few
-                        # candidates twice (27 % at 1M x 768): no distance cache, the sketch alone
-                        first = BEAM_NO_CACHE if (loop == 0 and self.circulant_start) else 0
+                        # candidates twice (27 % at 1M x 768): with short sketch rows the cache's probes cost
+                        # more than those repeats save, with long ones less (per launch, without and with the
+                        # cache: 0.36 and 0.39 ms at 384 columns, 0.73 and 0.68 ms at 768, 1.54 and 1.28 ms at 1536)
+                        first = BEAM_NO_CACHE if (loop == 0 and self.circulant_start and vectors.size(1) <= 512) else 0
                         t = search(vectors[start:end], queue, vectors, self.beams, config, exclude, flags=first,
                                    sketch=self.sketch)
                     else:
