@@ -253,6 +253,19 @@ int64_t vl_sketch_row_bytes(int64_t dim);
 int vl_sketch_build(const float *vectors, int64_t n_vectors, int64_t dim,
                     uint8_t *table, void *stream);
 
+/* Bounds of gathered cosine distances from the sketch: for every id
+ * lo[r, j] <= d(queries[r], vectors[ids[r, j]]) <= hi[r, j], where d is the very
+ * float32 value vl_gather_distances returns (VL_MAXFLOAT twice for an empty or
+ * out-of-range id).  The code that the beam-search step runs on its
+ * candidates, exposed so that the bound can be checked on its own.  workspace:
+ * vl_sketch_bounds_workspace_bytes(n_rows, dim) bytes, 16-byte aligned (the
+ * query rows rounded to 15 bits).  dim: a multiple of 4, at most 2048. */
+int64_t vl_sketch_bounds_workspace_bytes(int64_t n_rows, int64_t dim);
+int vl_sketch_bounds(const float *queries, int64_t n_rows, int64_t dim,
+                     const uint8_t *table, int64_t n_vectors,
+                     const int32_t *ids, int64_t m, float *lo, float *hi,
+                     void *workspace, int64_t workspace_bytes, void *stream);
+
 /* vl_closest_vectors with the sketch of `vectors` (NULL: exactly
  * vl_closest_vectors).  Same arguments, same result, same return value.  The
  * sketch serves the fused step under the cosine metric for 16-byte aligned rows

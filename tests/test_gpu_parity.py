@@ -1150,3 +1150,66 @@ def test_build_with_and_without_the_sketch():
         ann = ANN(gv, sketch=sketch, **kw)
         assert np.array_equal(host(ann.beams), wb), sketch
         assert np.array_equal(bits(host(ann.distances)), bits(wd)), sketch
+
+
+@pytest.mark.parametrize("dim", [4, 64, 100, 128, 256, 384, 512, 768, 1024, 1536, 2048])
+def test_sketch_bounds_hold_for_the_exact_kernel(dim):
+    """vl_sketch_bounds (the code the beam-search step runs on its candidates): lo <= d <= hi for the float32
+    distance the exact kernel returns, on random pairs and on the pairs that stress the bound - a query along
+    what the rounding moved (the Cauchy-Schwarz worst case, both signs), a query equal or opposite to the row,
+    a query with one huge and many tiny elements (coarse steps of its own rounding), rows that are not of unit
+    length, rows of zeros, tiny rows, NaN.  And the bounds are worth something: on unit rows hi - lo stays
+    within 2.3 x ||q|| x (what the rounding moved)."""
+    say(f"sketch bounds dim={dim}")
+    from vectorlink_gpu.kernels import build_sketch, gather_distances, sketch_bounds, sketch_row_bytes
+
+    rng = np.random.default_rng(1000 + dim)
+    n, nq, m = 600, 96, 200
+    v = unit(rng, n, dim)
+    v[1] = 0.0
+    v[2] *= 6.5
+    v[4] = np.float32(1e-30) * v[4]
+    v[5] *= 0.01
+    sk = build_sketch(dev(v))
+    t = host(sk)
+    pad = sketch_row_bytes(dim) - 16
+    u = t[:, :dim].view(np.int8).astype(np.float64)
+    tail = t[:, pad:].copy().view(np.float32)
+    moved = v.astype(np.float64) - tail[:, :1].astype(np.float64) * u       # what the rounding moved, per row
+    q = unit(rng, nq, dim)
+    ids = rng.integers(0, n, (nq, m)).astype(np.int32)
+    ids[:, 0] = np.arange(nq) + 10
+    for r in range(0, 24):                                                   # along / against the moved part
+        e = moved[ids[r, 0]]
+        if np.linalg.norm(e) > 0:
+            q[r] = (e / np.linalg.norm(e) * (1 if r % 2 else -1)).astype(np.float32)
+    for r in range(24, 36):
+        q[r] = v[ids[r, 0]] * (1 if r % 2 else -1)                           # the row itself / its opposite
+    for r in range(36, 48):
+        q[r] = (rng.standard_normal(dim) * 1e-3).astype(np.float32)
+        q[r, r % dim] = 1.0                                                  # one big element: coarse steps
+    q[48] *= 3.0                                                             # queries that are not unit length
+    q[49] = 0.0
+    q[50] = np.float32(1e-32) * q[50]
+    ids[:, 5] = M
+    ids[:, 6] = n + 7                                                        # out of range
+    (lo, hi) = sketch_bounds(dev(q), sk, dev(ids))
+    d = host(gather_distances(dev(q), dev(v), dev(np.where(ids >= n, M, ids).astype(np.int32))))
+    lo, hi = host(lo), host(hi)
+    empty = (ids == M) | (ids >= n)
+    assert np.all(lo[empty] == np.float32(F)) and np.all(hi[empty] == np.float32(F))
+    real = ~empty
+    assert np.all(lo[real] <= d[real]) and np.all(d[real] <= hi[real])
+    # not vacuous: on unit queries and unit rows the gap is about 2 eps = ||q|| x moved (in distance units: / 2 x 2)
+    rows = np.arange(51, nq)
+    cols = np.arange(7, m)
+    sub = ids[np.ix_(rows, cols)]
+    unit_rows = np.isin(sub, [1, 2, 4, 5], invert=True)
+    gap = (hi - lo)[np.ix_(rows, cols)][unit_rows]
+    want = np.linalg.norm(moved[sub[unit_rows]], axis=1)
+    assert np.all(gap <= 2.3 * want * 0.5 * 2 + 1e-5) and np.all(gap > 0)
+    # a query with a NaN: nothing is promised, and nothing wrong is claimed (lo <= hi or a NaN)
+    q[0, 0] = np.nan
+    (lo2, hi2) = sketch_bounds(dev(q[:1]), sk, dev(ids[:1]))
+    lo2, hi2 = host(lo2)[0][real[0]], host(hi2)[0][real[0]]
+    assert np.all(np.isnan(lo2) | np.isnan(hi2) | ((lo2 == 0) & (hi2 == 1)))

@@ -120,6 +120,48 @@ __global__ __launch_bounds__(256) void sketch_query_kernel(const float *__restri
     }
 }
 
+// Bounds of gathered distances: one workgroup per query row, a wavefront per 64 ids; the very code
+// (sketch_query_load, wave_sketch) the beam-search step runs.
+template <int SCPL, int SLPR>
+__global__ __launch_bounds__(256) void sketch_bounds_kernel(const uint8_t *__restrict__ rounded, int64_t rounded_bytes,
+                                                            int chunks, const uint8_t *__restrict__ table,
+                                                            int64_t row_bytes, int64_t n_vectors,
+                                                            const int32_t *__restrict__ ids, int m, int64_t row0,
+                                                            float *__restrict__ lo, float *__restrict__ hi) {
+    const int64_t row = row0 + blockIdx.x;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    __shared__ float out_lo[256 / kWave][kWave], out_hi[256 / kWave][kWave];
+    SketchQuery<SCPL> sq;
+    sketch_query_load<SCPL, SLPR>(sq, rounded + row * rounded_bytes, chunks);
+    for (int c0 = wave * kWave; c0 < m; c0 += 256) {
+        const int slot = c0 + lane;
+        const int32_t id = slot < m ? ids[row * m + slot] : VL_MAXINT;
+        const bool ok = slot < m && id != VL_MAXINT && id >= 0 && (int64_t)id < n_vectors;
+        out_lo[wave][lane] = VL_MAXFLOAT;
+        out_hi[wave][lane] = VL_MAXFLOAT;
+        wave_sketch<SCPL, SLPR, 2>(sq, table, row_bytes, chunks, id, ok, out_lo[wave], out_hi[wave]);
+        // (the wavefront's own LDS writes and reads are in program order)
+        if (slot < m) {
+            lo[row * m + slot] = out_lo[wave][lane];
+            hi[row * m + slot] = out_hi[wave][lane];
+        }
+    }
+}
+
+template <int SCPL, int SLPR>
+int launch_sketch_bounds(const uint8_t *rounded, int64_t dim, const uint8_t *table, int64_t n_vectors, const int32_t *ids,
+                         int64_t n_rows, int64_t m, float *lo, float *hi, hipStream_t st) {
+    for (int64_t row0 = 0; row0 < n_rows; row0 += kMaxBlocks) {
+        int64_t rows = n_rows - row0 < kMaxBlocks ? n_rows - row0 : kMaxBlocks;
+        hipLaunchKernelGGL((sketch_bounds_kernel<SCPL, SLPR>), dim3((unsigned)rows), dim3(256), 0, st, rounded,
+                           sketch_query_bytes(dim), (int)sketch_data_chunks(dim), table, sketch_row_bytes(dim), n_vectors,
+                           ids, (int)m, row0, lo, hi);
+        VL_LAUNCH_CHECK("sketch_bounds_kernel");
+    }
+    return VL_OK;
+}
+
 }  // namespace
 
 // Rounded query rows for a beam-search call that uses the sketch; out_rows: n_rows x sketch_query_bytes(dim),
@@ -155,4 +197,37 @@ VL_EXPORT int vl_sketch_build(const float *vectors, int64_t n_vectors, int64_t d
         VL_LAUNCH_CHECK("sketch_build_kernel");
     }
     return VL_OK;
+}
+
+VL_EXPORT int64_t vl_sketch_bounds_workspace_bytes(int64_t n_rows, int64_t dim) {
+    if (n_rows < 0 || dim <= 0) {
+        vl_set_error("bad sizes");
+        return VL_ERR_ARG;
+    }
+    return n_rows * sketch_query_bytes(dim) + 256;
+}
+
+VL_EXPORT int vl_sketch_bounds(const float *queries, int64_t n_rows, int64_t dim, const uint8_t *table,
+                               int64_t n_vectors, const int32_t *ids, int64_t m, float *lo, float *hi,
+                               void *workspace, int64_t workspace_bytes, void *stream) {
+    VL_REQUIRE(n_rows >= 0 && m >= 0 && n_vectors >= 0 && dim > 0, "bad sizes");
+    if (n_rows == 0 || m == 0) return VL_OK;
+    VL_REQUIRE(queries && table && ids && lo && hi && workspace, "null pointer");
+    VL_REQUIRE(dim % 4 == 0 && dim <= 2048 && ((uintptr_t)queries & 15) == 0 && ((uintptr_t)table & 15) == 0,
+               "the sketch serves 16-byte aligned rows of up to 2048 columns, a multiple of 4");
+    VL_REQUIRE(((uintptr_t)workspace & 15) == 0 && workspace_bytes >= n_rows * sketch_query_bytes(dim),
+               "workspace too small or not 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    uint8_t *rounded = (uint8_t *)workspace;
+    int rc = vl_launch_sketch_queries(queries, n_rows, dim, rounded, st);
+    if (rc < 0) return rc;
+    const int chunks = (int)sketch_data_chunks(dim);
+    if (chunks <= 8) return launch_sketch_bounds<1, 8>(rounded, dim, table, n_vectors, ids, n_rows, m, lo, hi, st);
+    if (chunks <= 16) return launch_sketch_bounds<2, 8>(rounded, dim, table, n_vectors, ids, n_rows, m, lo, hi, st);
+    if (chunks <= 24) return launch_sketch_bounds<3, 8>(rounded, dim, table, n_vectors, ids, n_rows, m, lo, hi, st);
+    if (chunks <= 32) return launch_sketch_bounds<2, 16>(rounded, dim, table, n_vectors, ids, n_rows, m, lo, hi, st);
+    if (chunks <= 48) return launch_sketch_bounds<3, 16>(rounded, dim, table, n_vectors, ids, n_rows, m, lo, hi, st);
+    if (chunks <= 64) return launch_sketch_bounds<4, 16>(rounded, dim, table, n_vectors, ids, n_rows, m, lo, hi, st);
+    if (chunks <= 96) return launch_sketch_bounds<3, 32>(rounded, dim, table, n_vectors, ids, n_rows, m, lo, hi, st);
+    return launch_sketch_bounds<4, 32>(rounded, dim, table, n_vectors, ids, n_rows, m, lo, hi, st);
 }

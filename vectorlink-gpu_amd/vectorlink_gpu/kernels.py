@@ -197,6 +197,26 @@ def build_sketch(vectors: Tensor) -> Tensor:
     return out
 
 
+def sketch_bounds(queries: Tensor, sketch: Tensor, ids: Tensor) -> Tuple[Tensor, Tensor]:
+    """(lo, hi) with lo[r, j] <= gather_distances(queries, vectors, ids)[r, j] <= hi[r, j], from the 8-bit sketch
+    of `vectors` alone (no counterpart in the reference): what a beam-search row knows of a candidate before it
+    decides whether to fetch it."""
+    _check_f32(queries, "queries")
+    _check_ids(ids, "ids")
+    nv.require_gpu(queries, sketch, ids)
+    assert sketch.dtype == torch.uint8 and sketch.is_contiguous()
+    (rows, m) = ids.size()
+    dim = queries.size(1)
+    assert queries.size(0) == rows and sketch.size(1) == sketch_row_bytes(dim)
+    lo = torch.empty((rows, m), dtype=torch.float32, device=ids.device)
+    hi = torch.empty((rows, m), dtype=torch.float32, device=ids.device)
+    need = nv.check(nv.lib().vl_sketch_bounds_workspace_bytes(rows, dim))
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=ids.device)
+    nv.check(nv.lib().vl_sketch_bounds(nv.ptr(queries), rows, dim, nv.ptr(sketch), sketch.size(0), nv.ptr(ids), m,
+                                       nv.ptr(lo), nv.ptr(hi), nv.ptr(ws), ws.numel(), nv.stream()))
+    return (lo, hi)
+
+
 def optimize_graph(beams: Tensor, degree: int) -> Tensor:
     """Rank-based graph optimisation (not in the reference): re-order every row of
     `beams` ([N, W], best first, MAXINT = empty) by the number of two-hop detours
