@@ -365,6 +365,43 @@ __device__ inline uint64_t block_min_key(uint64_t mine, uint64_t *red, int round
     return m;
 }
 
+// Smallest 32-bit value over a wavefront, in every lane: halves and rows are folded with the swap instructions
+// and DPP row shifts that fold_group uses (a lane without a source keeps its own value), a few cycles per
+// step where a cross-lane shuffle through the LDS crossbar takes a round trip each.
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t x) {
+    {
+        uint32_t lo = x, hi = x;
+        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+        x = lo < hi ? lo : hi;
+    }
+    {
+        uint32_t even = x, odd = x;
+        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(even), "+v"(odd));
+        x = even < odd ? even : odd;
+    }
+    uint32_t y;
+    y = __builtin_amdgcn_update_dpp(x, x, 0x108, 0xf, 0xf, false); x = y < x ? y : x;  // row_shl:8
+    y = __builtin_amdgcn_update_dpp(x, x, 0x104, 0xf, 0xf, false); x = y < x ? y : x;  // row_shl:4
+    y = __builtin_amdgcn_update_dpp(x, x, 0x102, 0xf, 0xf, false); x = y < x ? y : x;  // row_shl:2
+    y = __builtin_amdgcn_update_dpp(x, x, 0x101, 0xf, 0xf, false); x = y < x ? y : x;  // row_shl:1
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)x);
+}
+
+// Smallest value over the workgroup of each thread's `mine` (0xFFFFFFFF = none).
+// red: 2 * kQueueWaves words of LDS, used alternately so one barrier per call suffices.
+__device__ inline uint32_t block_min_u32(uint32_t mine, uint32_t *red, int round) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int nw = blockDim.x / kWave;
+    mine = wave_min_u32(mine);
+    uint32_t *slot = red + (round & 1) * kQueueWaves;
+    if (lane == 0) slot[wave] = mine;
+    __syncthreads();
+    uint32_t m = slot[0];
+    for (int w = 1; w < nw; ++w) m = slot[w] < m ? slot[w] : m;
+    return m;
+}
+
 // Workgroup-wide scalars shared by the expand and merge phases of a row.
 __shared__ int g_n_ex_s;                  // exclusion ids before the row's first empty one
 __shared__ int32_t g_visit_s[kMaxVisit];  // the ids popped from the visit queue in this iteration
@@ -538,25 +575,32 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
         }
         fl[i] = f;
     }
-    uint64_t sel_max = 0ull;  // largest selected key among the "rest" candidates
+    // The Vt smallest distinct keys among the "rest" candidates are found by their distances alone (the high
+    // word of a key): Vt rounds of a workgroup-wide minimum over 32-bit words give the Vt smallest distinct
+    // distances, and every "rest" candidate at or below the last of them is taken - the same candidates, plus
+    // others of equal distance when there are ties, which the merges below cut by rank.
+    uint32_t sel_max = 0u;  // largest selected distance word among the "rest" candidates
+    bool any_rest = false;
     if (!seen_full) {
-        uint64_t last = wv;
+        uint32_t *red32 = reinterpret_cast<uint32_t *>(red);
+        uint32_t last = 0u;
         for (int r = 0; r < a.Vt; ++r) {
-            uint64_t mine = kPadKey;
+            uint32_t mine = 0xFFFFFFFFu;
             for (int i = threadIdx.x; i < a.m; i += blockDim.x) {
-                uint64_t k = raw[i];
-                if ((fl[i] & 2) && k > last && k < mine) mine = k;
+                const uint32_t k = (uint32_t)(raw[i] >> 32);
+                if ((fl[i] & 2) && (r == 0 || k > last) && k < mine) mine = k;
             }
-            uint64_t mn = block_min_key(mine, red, r);
-            if (mn == kPadKey) break;
+            const uint32_t mn = block_min_u32(mine, red32, r);
+            if (mn == 0xFFFFFFFFu) break;
             last = mn;
             sel_max = mn;
+            any_rest = true;
         }
     }
     __syncthreads();
     auto wanted = [&](int i) -> bool {
         uint8_t f = fl[i];
-        return (f & 1) || ((f & 2) && raw[i] <= sel_max);
+        return (f & 1) || (any_rest && (f & 2) && (uint32_t)(raw[i] >> 32) <= sel_max);
     };
     const int n_u = block_compact(raw, a.m, uk, wanted, wave_cnt);
     int Pu = 2;
