@@ -46,7 +46,7 @@ MFMA_FP32_PEAK = 157.3  # MI355X published dense fp32 matrix TFLOP/s
 # (FETCH_SIZE x 2.0 after calibration against the 1 GiB copy + WRITE_SIZE x 1.0, "roofline pass" phases);
 # NOT measured in this run.  Workloads without a recorded counter run report null.
 TRAFFIC_PER_LOOP = {
-    "mix-1m-768": [(2201215.4 * 2 + 159395.8) * 1024, (807213.5 * 2 + 61046.3) * 1024, (416360.8 * 2 + 25897.5) * 1024],
+    "mix-1m-768": [(2201808.1 * 2 + 159398.8) * 1024, (807559.1 * 2 + 61049.6) * 1024, (416786.9 * 2 + 25897.2) * 1024],
     "mix-1m-128": [(436666.3 * 2 + 25910.0) * 1024, (231534.4 * 2 + 28947.1) * 1024, (153222.4 * 2 + 20410.1) * 1024],
 }
 

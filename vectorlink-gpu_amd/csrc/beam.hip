@@ -352,10 +352,33 @@ __device__ inline uint64_t block_min_key(uint64_t mine, uint64_t *red, int round
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const int nw = blockDim.x / kWave;
-#pragma unroll
-    for (int h = kWave / 2; h >= 1; h >>= 1) {
-        uint64_t o = __shfl_xor((unsigned long long)mine, h);
-        mine = o < mine ? o : mine;
+    {
+        // folded like wave_min_u32 below, both words of a key moving together; lane 0 ends with the minimum
+        uint32_t lo = (uint32_t)mine, hi = (uint32_t)(mine >> 32);
+        auto take = [&](uint32_t olo, uint32_t ohi) {
+            const bool less = ohi < hi || (ohi == hi && olo < lo);
+            lo = less ? olo : lo;
+            hi = less ? ohi : hi;
+        };
+        {
+            uint32_t a0 = lo, a1 = lo, b0 = hi, b1 = hi;
+            asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\tv_permlane32_swap_b32 %2, %3\n\ts_nop 1"
+                         : "+v"(a0), "+v"(a1), "+v"(b0), "+v"(b1));
+            lo = a0; hi = b0;
+            take(a1, b1);
+        }
+        {
+            uint32_t a0 = lo, a1 = lo, b0 = hi, b1 = hi;
+            asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\tv_permlane16_swap_b32 %2, %3\n\ts_nop 1"
+                         : "+v"(a0), "+v"(a1), "+v"(b0), "+v"(b1));
+            lo = a0; hi = b0;
+            take(a1, b1);
+        }
+        take(__builtin_amdgcn_update_dpp(lo, lo, 0x108, 0xf, 0xf, false), __builtin_amdgcn_update_dpp(hi, hi, 0x108, 0xf, 0xf, false));
+        take(__builtin_amdgcn_update_dpp(lo, lo, 0x104, 0xf, 0xf, false), __builtin_amdgcn_update_dpp(hi, hi, 0x104, 0xf, 0xf, false));
+        take(__builtin_amdgcn_update_dpp(lo, lo, 0x102, 0xf, 0xf, false), __builtin_amdgcn_update_dpp(hi, hi, 0x102, 0xf, 0xf, false));
+        take(__builtin_amdgcn_update_dpp(lo, lo, 0x101, 0xf, 0xf, false), __builtin_amdgcn_update_dpp(hi, hi, 0x101, 0xf, 0xf, false));
+        mine = ((uint64_t)hi << 32) | lo;
     }
     uint64_t *slot = red + (round & 1) * kQueueWaves;
     if (lane == 0) slot[wave] = mine;
