@@ -47,7 +47,7 @@ MFMA_FP32_PEAK = 157.3  # MI355X published dense fp32 matrix TFLOP/s
 # NOT measured in this run.  Workloads without a recorded counter run report null.
 TRAFFIC_PER_LOOP = {
     "mix-1m-768": [(2201808.1 * 2 + 159398.8) * 1024, (807559.1 * 2 + 61049.6) * 1024, (416786.9 * 2 + 25897.2) * 1024],
-    "mix-1m-128": [(436666.3 * 2 + 25910.0) * 1024, (231534.4 * 2 + 28947.1) * 1024, (153222.4 * 2 + 20410.1) * 1024],
+    "mix-1m-128": [(436762.3 * 2 + 25917.2) * 1024, (231523.9 * 2 + 28948.6) * 1024, (153260.6 * 2 + 20410.3) * 1024],
 }
 
 
