@@ -1213,3 +1213,34 @@ def test_sketch_bounds_hold_for_the_exact_kernel(dim):
     (lo2, hi2) = sketch_bounds(dev(q[:1]), sk, dev(ids[:1]))
     lo2, hi2 = host(lo2)[0][real[0]], host(hi2)[0][real[0]]
     assert np.all(np.isnan(lo2) | np.isnan(hi2) | ((lo2 == 0) & (hi2 == 1)))
+
+
+def test_search_with_the_sketch_equals_the_oracle():
+    """ANN.search(sketch=True): the same queues as the oracle's search, under both seedings and both stops."""
+    say("search with the sketch, n=2500 dim=256")
+    from vectorlink_gpu import ANN
+
+    rng = np.random.default_rng(99)
+    n, dim, nq = 2500, 256, 200
+    centres = rng.standard_normal((25, dim)).astype(np.float32)
+    v = centres[rng.integers(0, 25, n)] + 0.15 * rng.standard_normal((n, dim)).astype(np.float32)
+    v = (v / np.linalg.norm(v, axis=1, keepdims=True)).astype(np.float32)
+    q = centres[rng.integers(0, 25, nq)] + 0.15 * rng.standard_normal((nq, dim)).astype(np.float32)
+    q = (q / np.linalg.norm(q, axis=1, keepdims=True)).astype(np.float32)
+    kw = dict(beam_size=16, beam_queue_factor=2, batch_size=900, optimization_loops=2)
+    c = cfg(**kw)
+    (wb, _) = orc.generate_ann(v, c)
+    ann = ANN(dev(v), **kw)
+    assert np.array_equal(host(ann.beams), wb)
+    for stop in ("batch", "per_query"):
+        want = orc.search(v, wb, q, c, stop=stop)
+        L = want.length
+        for use in (True, False):
+            got = ann.search(dev(q), stop=stop, sketch=use)
+            assert np.array_equal(host(got.indices)[:, :L], want.indices[:, :L]), (stop, use)
+            assert np.array_equal(bits(host(got.distances)[:, :L]), bits(want.distances[:, :L])), (stop, use)
+    # dense seeds: no oracle for the seeding tiles' choice, so the two paths are compared with each other
+    a = ann.search(dev(q), seeding="dense", sketch=True)
+    b = ann.search(dev(q), seeding="dense", sketch=False)
+    assert torch.equal(a.indices[:, :a.length], b.indices[:, :b.length])
+    assert torch.equal(a.distances[:, :a.length].view(torch.int32), b.distances[:, :b.length].view(torch.int32))

@@ -540,6 +540,7 @@ class ANN:
         assert seed_dims is None or (seed_dims > 0 and seed_dims % 4 == 0), "seed_dims must be a multiple of 4"
         self._entry = None
         self._queues = None
+        self._sketch = None   # the 8-bit sketch of the vectors, when the build made one (or a search asked for it)
         (count, dim) = vectors.size()
         self.configuration: Dict = {
             "prune": prune,
@@ -572,6 +573,7 @@ class ANN:
             for _ in build.steps():
                 pass
             self.build_stats: list = build.stats
+            self._sketch = build.sketch
             (self.beams, self.distances) = build.result()
             if keep_queues:
                 width = build.beams.size(1)
@@ -655,8 +657,19 @@ class ANN:
             self._entry = (ids, rows.contiguous())
         return self._entry
 
+    def _search_sketch(self, use: bool) -> Optional[Tensor]:
+        """The sketch for a search that asks for one (made now if the build did not make it)."""
+        dim = self.vectors.size(1)
+        able = (self.configuration.get("sketch", True) and self.configuration.get("metric", "cosine") == "cosine"
+                and dim % 4 == 0 and dim <= 2048)
+        if not (use and able):
+            return None
+        if self._sketch is None:
+            self._sketch = build_sketch(self.vectors)
+        return self._sketch
+
     def search(self, query: Tensor, queue_size: Optional[int] = None, seeding: Optional[str] = None,
-               stop: str = "batch") -> Queue:
+               stop: str = "batch", sketch: bool = False) -> Queue:
         """reference ann.py:469-477: takes a batch of query vectors, returns the
         search Queue; the answer is queue.indices[:, :k] / queue.distances[:, :k].
         queue_size overrides the configured search-queue length, seeding the
@@ -664,7 +677,12 @@ class ANN:
         expands until no row of the batch changed at a progress check);
         stop="per_query" finishes each row on its own after speculative_readahead
         iterations in a row that left its queue unchanged - faster for large
-        batches, not the reference's result."""
+        batches, not the reference's result.  sketch=True (an addition) lets the
+        search decide from the 8-bit sketch of the vectors which candidate rows to
+        fetch; the result is the same.  Off by default: a search runs on the pruned
+        graph, whose candidates are near neighbours the sketch cannot tell apart, so
+        its rows give the sketch up after a few iterations (measured: 64 k QPS
+        either way at 1M x 1536, 120 k without and 116 k with it at 1M x 768)."""
         assert stop in ("batch", "per_query")
         assert query.dim() == 2 and query.dtype == torch.float32
         if not query.is_cuda:
@@ -679,7 +697,7 @@ class ANN:
         else:
             search_queue = initial_search_queue(self.vectors, query, self.configuration, queue_size)
         closest_vectors(query, search_queue, self.vectors, self.beams, self.configuration, None,
-                        flags=BEAM_PER_QUERY_STOP if stop == "per_query" else 0)
+                        flags=BEAM_PER_QUERY_STOP if stop == "per_query" else 0, sketch=self._search_sketch(sketch))
         return search_queue
 
     def recall_at_k(self, query: Tensor, k: int = 10, queue_size: Optional[int] = None,
