@@ -574,7 +574,8 @@ def test_closest_vectors_seeded_configuration_sweep():
     shapes with and without slack, exclusion lists of several columns, search- and
     build-shaped calls) through the fused loop against the oracle."""
     from vectorlink_gpu import Queue
-    from vectorlink_gpu.ann import closest_vectors
+    from vectorlink_gpu.ann import BEAM_NO_CACHE, closest_vectors
+    from vectorlink_gpu.kernels import build_sketch
 
     master = np.random.default_rng(2025)
     for case in range(40):
@@ -616,6 +617,17 @@ def test_closest_vectors_seeded_configuration_sweep():
         assert t_got == t_want, case
         assert np.array_equal(host(gq.indices)[:, :length], oq.indices[:, :length]), case
         assert np.array_equal(bits(host(gq.distances)[:, :length]), bits(oq.distances[:, :length])), case
+        if dim % 4 == 0:
+            # the same call through the 8-bit sketch of the vectors, with and without the distance cache
+            sk = build_sketch(dev(v))
+            for flags in (0, BEAM_NO_CACHE):
+                gq = Queue(b, length, cap)
+                gq.insert(dev(seeds), dev(sd))
+                t_got = closest_vectors(dev(q), gq, dev(v), dev(table), c, None if ex is None else dev(ex), flags=flags,
+                                        sketch=sk)
+                assert t_got == t_want, (case, flags)
+                assert np.array_equal(host(gq.indices)[:, :length], oq.indices[:, :length]), (case, flags)
+                assert np.array_equal(bits(host(gq.distances)[:, :length]), bits(oq.distances[:, :length])), (case, flags)
 
 
 def test_command_line_driver_and_parameter_sweep(tmp_path):
