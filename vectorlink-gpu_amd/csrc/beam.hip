@@ -1380,7 +1380,7 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     if (step.memo) {
         int lg = 0;
         while ((1 << lg) < l.memo_slots) ++lg;
-        VL_REQUIRE((1 << lg) == l.memo_slots, "memo slots must be a power of two");
+        VL_REQUIRE((1 << lg) == l.memo_slots && lg >= 4, "memo slots must be a power of two, 16 or more");
         step.memo_shift = 32 - lg;
     }
     // with a sketch every row starts out using it (and the cache, when there is one)

@@ -177,7 +177,7 @@ int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors,
     if (a.memo) {
         int lg = 0;
         while ((1 << lg) < memo_slots) ++lg;
-        VL_REQUIRE((1 << lg) == memo_slots && lg >= 1 && lg <= 24, "memo slots must be a power of two");
+        VL_REQUIRE((1 << lg) == memo_slots && lg >= 4 && lg <= 24, "memo slots must be a power of two, 16 or more");
         a.memo_shift = 32 - lg;
     }
     a.n_rows = n_rows; a.n_vectors = n_vectors; a.n_nodes = n_nodes;

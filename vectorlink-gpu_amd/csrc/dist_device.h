@@ -22,7 +22,13 @@ __device__ __forceinline__ float finish_distance(float sum, bool l2) { return l2
 // table concurrently, so an entry is always moved as ONE relaxed 64-bit atomic
 // access: a reader sees a whole entry (old or new), never the id of one and the
 // distance of another.
-__device__ __forceinline__ uint32_t memo_hash(int32_t id, int shift) { return ((uint32_t)id * 2654435761u) >> shift; }
+// The 16 ids of an aligned group share a 128-byte line of the table (the group is hashed, the id's low four bits
+// pick the entry within it): neighbour lists of a graph with local structure, such as the circulant graph a
+// build starts from, probe and fill a few lines instead of one per candidate.  Tables have at least 16 slots.
+__device__ __forceinline__ uint32_t memo_hash(int32_t id, int shift) {
+    const uint32_t group = (((uint32_t)id >> 4) * 2654435761u) >> shift;
+    return (group & ~15u) | ((uint32_t)id & 15u);
+}
 __device__ __forceinline__ void memo_store(uint64_t *memo_row, int shift, int32_t id, float d) {
     uint64_t e = ((uint64_t)__builtin_bit_cast(uint32_t, d) << 32) | (uint32_t)id;
     __hip_atomic_store(memo_row + memo_hash(id, shift), e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
