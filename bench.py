@@ -46,8 +46,8 @@ MFMA_FP32_PEAK = 157.3  # MI355X published dense fp32 matrix TFLOP/s
 # (FETCH_SIZE x 2.0 after calibration against the 1 GiB copy + WRITE_SIZE x 1.0, "roofline pass" phases);
 # NOT measured in this run.  Workloads without a recorded counter run report null.
 TRAFFIC_PER_LOOP = {
-    "mix-1m-768": [(2201808.1 * 2 + 159398.8) * 1024, (807559.1 * 2 + 61049.6) * 1024, (416786.9 * 2 + 25897.2) * 1024],
-    "mix-1m-128": [(436762.3 * 2 + 25917.2) * 1024, (231523.9 * 2 + 28948.6) * 1024, (153260.6 * 2 + 20410.3) * 1024],
+    "mix-1m-768": [(2072185.7 * 2 + 155367.1) * 1024, (806583.7 * 2 + 61026.9) * 1024, (417181.9 * 2 + 25924.5) * 1024],
+    "mix-1m-128": [(430414.2 * 2 + 25794.5) * 1024, (231365.9 * 2 + 28947.2) * 1024, (153333.9 * 2 + 20416.3) * 1024],
 }
 
 

@@ -266,7 +266,7 @@ class GraphBuild:
                         # the neighbour lists of a circulant graph share little, so a search of it meets few
                         # candidates twice (27 % at 1M x 768): with short sketch rows the cache's probes cost
                         # more than those repeats save, with long ones less (per launch, without and with the
-                        # cache: 0.36 and 0.39 ms at 384 columns, 0.73 and 0.68 ms at 768, 1.54 and 1.28 ms at 1536)
+                        # cache: 0.35 and 0.37 ms at 384 columns, 0.73 and 0.64 ms at 768, 1.54 and 1.24 ms at 1536)
                         first = BEAM_NO_CACHE if (loop == 0 and self.circulant_start and vectors.size(1) <= 512) else 0
                         t = search(vectors[start:end], queue, vectors, self.beams, config, exclude, flags=first,
                                    sketch=self.sketch)
