@@ -65,11 +65,11 @@ def profile_read(nv, reset=True, enable=1):
 
 def step_roofline(prof, dim, batch_rows):
     """Algorithmic bytes of the beam-search step from the hook counters: 4*dim + 12 per candidate row actually
-    fetched and evaluated, a sketch row + the id (16*ceil(dim/16) + 16 + 4) per candidate looked at through the
+    fetched and evaluated, a sketch row, its tail and the id (16*ceil(dim/16) + 8 + 4) per candidate looked at through the
     8-bit sketch, plus the query row (4*dim) once per (row, iteration)."""
     launches = max(prof["expand_launches"], 1.0)
     per_eval = 4 * dim + 12
-    per_sketch = 16 * ((dim + 15) // 16) + 16 + 4
+    per_sketch = 16 * ((dim + 15) // 16) + 8 + 4
     q_loads = prof["iterations"] * batch_rows * 4.0 * dim
     algo = prof["evals"] * per_eval + prof["sketched"] * per_sketch + q_loads
     secs = prof["expand_ms"] / 1e3

@@ -231,11 +231,14 @@ int64_t vl_closest_vectors(const vl_beam_params *p,
  *
  * The reference evaluates every candidate distance of an iteration in full
  * (cuda_search_from_seeds_kernel, kernels.py:204-257) although a row keeps a
- * handful of its hundreds of candidates.  A sketch row holds the vector rounded
- * to 8 bits per element with one scale per row (dim int8 values round(v / scale),
- * scale = max |v| / 127, padded with zeros to a multiple of 16) and a 16-byte
- * tail: float scale, float bound on the 2-norm of what the rounding moved, float
- * bound on the row's 2-norm, float 0.  With it a dot product is known to within
+ * handful of its hundreds of candidates.  The sketch holds every vector rounded
+ * to 8 bits per element with one scale per vector (dim int8 values round(v / scale),
+ * scale = max |v| / 127, padded with zeros to a multiple of 16) and an 8-byte
+ * tail: float scale, then as halves, rounded up, a bound on the 2-norm of what
+ * the rounding moved and a bound on the vector's 2-norm.  The table is ONE block:
+ * the n_vectors data rows first (16 * ceil(dim / 16) bytes each), then the
+ * n_vectors tails - a part of it is not the sketch of a part of the vectors.
+ * With it a dot product is known to within
  * ||q|| x that bound (Cauchy-Schwarz) from a quarter of the bytes, by integer
  * arithmetic (the query row is rounded to 15 bits, which the bound accounts for).  vl_closest_vectors_with_sketch uses those bounds ONLY to decide
  * which candidate rows to fetch: a candidate whose lower bound is above the last
@@ -244,11 +247,12 @@ int64_t vl_closest_vectors(const vl_beam_params *p,
  * beyond it, cannot enter either queue and is dropped; every other candidate is
  * evaluated exactly.  Queues are bit-identical to vl_closest_vectors'. */
 
-/* Bytes per sketch row for vectors of `dim` columns: 16 * ceil(dim / 16) + 16. */
+/* Bytes per vector in the sketch of vectors of `dim` columns:
+ * 16 * ceil(dim / 16) + 8. */
 int64_t vl_sketch_row_bytes(int64_t dim);
 
-/* Fills table[n_vectors, vl_sketch_row_bytes(dim)] (16-byte aligned) from
- * vectors[n_vectors, dim].  A row holding a NaN or an infinity gets an infinite
+/* Fills table (n_vectors * vl_sketch_row_bytes(dim) bytes, 16-byte aligned; on a
+ * 128-byte boundary its rows cost least) from vectors[n_vectors, dim].  A row holding a NaN or an infinity gets an infinite
  * bound: its candidates are always evaluated exactly. */
 int vl_sketch_build(const float *vectors, int64_t n_vectors, int64_t dim,
                     uint8_t *table, void *stream);

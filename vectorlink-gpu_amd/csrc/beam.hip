@@ -743,7 +743,7 @@ struct StepArgs {
     int count_evals;
     int l2;  // 0: cosine distance, 1: squared L2
     const uint8_t *sketch;     // 8-bit sketch of `vectors` (sketch_device.h), or null
-    int64_t sketch_row_bytes;
+    const uint8_t *sketch_tails;  // the table's second part: 8 bytes per vector
     int sketch_chunks;         // 16-byte chunks of data in a sketch row
     const uint8_t *rounded_queries;  // the call's query rows rounded for the sketch (sketch_device.h)
     int64_t rounded_query_bytes;
@@ -934,7 +934,7 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
                     }
                 }
                 if (s.count_evals || resample) n_sketched += __popcll(__ballot(ok));
-                wave_sketch<SCPL, SLPR, SU>(sq, s.sketch, s.sketch_row_bytes, s.sketch_chunks, id, ok, ld + c0, le + c0,
+                wave_sketch<SCPL, SLPR, SU>(sq, s.sketch, s.sketch_tails, s.sketch_chunks, id, ok, ld + c0, le + c0,
                                             memo_row, s.memo_shift);
             }
             n_fetched = n_sketched;  // for the share of cache hits: what the cache did not answer
@@ -1374,7 +1374,7 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
                "a call with a sketch needs VL_BEAM_USES_SKETCH in flags (and a workspace sized with it)");
     step.rounded_queries = (const uint8_t *)(ws + l.off_rounded);
     step.rounded_query_bytes = sketch_query_bytes(p->dim);
-    step.sketch_row_bytes = sketch_row_bytes(p->dim);
+    step.sketch_tails = sketch ? sketch + sketch_tails_offset(p->n_vectors, p->dim) : nullptr;
     step.sketch_chunks = (int)sketch_data_chunks(p->dim);
     step.memo_shift = 32;
     if (step.memo) {

@@ -23,7 +23,7 @@ __global__ __launch_bounds__(256) void sketch_build_kernel(const float *__restri
     if (row >= n) return;
     const float *v = vectors + row * dim;
     const int chunks = (int)sketch_data_chunks(dim);
-    uint8_t *out = table + row * sketch_row_bytes(dim);
+    uint8_t *out = table + row * sketch_data_bytes(dim);
 
     float mx = 0.f;
     bool finite = true;
@@ -62,12 +62,12 @@ __global__ __launch_bounds__(256) void sketch_build_kernel(const float *__restri
         // scale * q by 2^-24 of |v_j|; the floor covers squares that underflow (elements below 1e-19);
         // a row that holds a NaN or an infinity promises nothing
         const float floor_ = 1.1e-19f * __builtin_sqrtf((float)dim);
-        float4 tail;
-        tail.x = finite ? scale : 0.f;
-        tail.y = finite ? __builtin_sqrtf(r2) * 1.001f + floor_ : __builtin_inff();
-        tail.z = finite ? __builtin_sqrtf(n2) * 1.001f + floor_ : __builtin_inff();
-        tail.w = 0.f;
-        *reinterpret_cast<float4 *>(out + (int64_t)chunks * 16) = tail;
+        const float resid = finite ? __builtin_sqrtf(r2) * 1.001f + floor_ : __builtin_inff();
+        const float norm = finite ? __builtin_sqrtf(n2) * 1.001f + floor_ : __builtin_inff();
+        uint2 tail;
+        tail.x = __builtin_bit_cast(uint32_t, finite ? scale : 0.f);
+        tail.y = half_bits_not_below(resid) | (half_bits_not_below(norm) << 16);
+        *reinterpret_cast<uint2 *>(table + sketch_tails_offset(n, dim) + row * kSketchTailBytes) = tail;
     }
 }
 
@@ -125,7 +125,7 @@ __global__ __launch_bounds__(256) void sketch_query_kernel(const float *__restri
 template <int SCPL, int SLPR>
 __global__ __launch_bounds__(256) void sketch_bounds_kernel(const uint8_t *__restrict__ rounded, int64_t rounded_bytes,
                                                             int chunks, const uint8_t *__restrict__ table,
-                                                            int64_t row_bytes, int64_t n_vectors,
+                                                            const uint8_t *__restrict__ tails, int64_t n_vectors,
                                                             const int32_t *__restrict__ ids, int m, int64_t row0,
                                                             float *__restrict__ lo, float *__restrict__ hi) {
     const int64_t row = row0 + blockIdx.x;
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(256) void sketch_bounds_kernel(const uint8_t *__res
         const bool ok = slot < m && id != VL_MAXINT && id >= 0 && (int64_t)id < n_vectors;
         out_lo[wave][lane] = VL_MAXFLOAT;
         out_hi[wave][lane] = VL_MAXFLOAT;
-        wave_sketch<SCPL, SLPR, 2>(sq, table, row_bytes, chunks, id, ok, out_lo[wave], out_hi[wave]);
+        wave_sketch<SCPL, SLPR, 2>(sq, table, tails, chunks, id, ok, out_lo[wave], out_hi[wave]);
         // (the wavefront's own LDS writes and reads are in program order)
         if (slot < m) {
             lo[row * m + slot] = out_lo[wave][lane];
@@ -155,7 +155,7 @@ int launch_sketch_bounds(const uint8_t *rounded, int64_t dim, const uint8_t *tab
     for (int64_t row0 = 0; row0 < n_rows; row0 += kMaxBlocks) {
         int64_t rows = n_rows - row0 < kMaxBlocks ? n_rows - row0 : kMaxBlocks;
         hipLaunchKernelGGL((sketch_bounds_kernel<SCPL, SLPR>), dim3((unsigned)rows), dim3(256), 0, st, rounded,
-                           sketch_query_bytes(dim), (int)sketch_data_chunks(dim), table, sketch_row_bytes(dim), n_vectors,
+                           sketch_query_bytes(dim), (int)sketch_data_chunks(dim), table, table + sketch_tails_offset(n_vectors, dim), n_vectors,
                            ids, (int)m, row0, lo, hi);
         VL_LAUNCH_CHECK("sketch_bounds_kernel");
     }

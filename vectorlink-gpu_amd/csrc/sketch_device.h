@@ -4,11 +4,14 @@
 // candidate matters only if its key is below the last slot of the search queue or of the visit queue,
 // or is one of the few best beyond that.  The sketch lets a row find out which candidates those are
 // for a quarter of the memory traffic.  A sketch row holds the vector rounded to 8 bits per element
-// with one scale per row, and how far that rounding moved the vector:
+// with one scale per row, and how far that rounding moved the vector.  The table of n vectors is one block
+// of n * sketch_row_bytes(dim) bytes in two parts, so that the rows of the first part start on 128-byte
+// lines whenever 16 * ceil(dim / 16) is a multiple of 128 (a row that straddles lines costs a line more than
+// its size: 903 instead of 788 bytes per candidate were measured past L2 at 768 columns with the tail in the row):
 //
-//   bytes [0, dim)            int8 u_j = round(v_j / scale), scale = max_j |v_j| / 127
-//   bytes [dim, pad16(dim))   0
-//   tail, 16 bytes            float scale; float resid >= ||v - scale u||_2; float norm >= ||v||_2; float 0
+//   data, n rows of 16 * ceil(dim / 16) bytes:   int8 u_j = round(v_j / scale), scale = max_j |v_j| / 127, then zeros
+//   tails, n entries of 8 bytes after the data:  float scale; half resid >= ||v - scale u||_2; half norm >= ||v||_2
+//                                                (both rounded up; sixteen neighbouring ids share a line)
 //
 // The query row is rounded too, to 15 bits per element (Q_j = round(q_j / qscale) = 128 qh_j + ql_j with
 // two int8 digits, qscale = max_j |q_j| / 16256), so that the sum is integer work, four elements per
@@ -26,7 +29,21 @@
 #include "dist_device.h"
 
 __host__ __device__ inline int64_t sketch_data_chunks(int64_t dim) { return (dim + 15) / 16; }
-__host__ __device__ inline int64_t sketch_row_bytes(int64_t dim) { return sketch_data_chunks(dim) * 16 + 16; }
+__host__ __device__ inline int64_t sketch_data_bytes(int64_t dim) { return sketch_data_chunks(dim) * 16; }
+constexpr int64_t kSketchTailBytes = 8;
+__host__ __device__ inline int64_t sketch_row_bytes(int64_t dim) { return sketch_data_bytes(dim) + kSketchTailBytes; }
+// where the tails of a table of n vectors start
+__host__ __device__ inline int64_t sketch_tails_offset(int64_t n, int64_t dim) { return n * sketch_data_bytes(dim); }
+
+__device__ __forceinline__ float half_bits_as_float(uint32_t h) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+// The smallest half that is not below x (x >= 0, or an infinity): bounds are stored rounded up.
+__device__ __forceinline__ uint32_t half_bits_not_below(float x) {
+    uint16_t h = __builtin_bit_cast(uint16_t, (_Float16)x);   // to nearest; beyond the largest half: infinity
+    if (half_bits_as_float(h) < x) ++h;                         // the next half up (from the largest one: infinity)
+    return h;
+}
 
 // Sum over a group of N neighbouring lanes, left in the group's first lane (other lanes end with
 // values nobody uses).  Same moves as fold_group, for groups of 8 lanes as well.
@@ -84,7 +101,7 @@ __device__ __forceinline__ void sketch_query_load(SketchQuery<SCPL> &sq, const u
 // instruction), a lane holds SCPL of its 16-byte chunks, SU loads of a group are in flight at a time.
 template <int SCPL, int SLPR, int SU>
 __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const uint8_t *__restrict__ table,
-                                            int64_t row_bytes, int data_chunks, int32_t my_id, bool ok,
+                                            const uint8_t *__restrict__ tails, int data_chunks, int32_t my_id, bool ok,
                                             float *__restrict__ out_lo, float *__restrict__ out_hi,
                                             uint64_t *memo_row = nullptr, int memo_shift = 0) {
     constexpr int G = kWave / SLPR;
@@ -96,7 +113,7 @@ __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const u
         int mysrc[SU];
         int32_t ids[SU];
         uint4 r[SU][SCPL];
-        float4 tail[SU];
+        uint2 tail[SU];
 #pragma unroll
         for (int u = 0; u < SU; ++u) {
             int s = -1;
@@ -112,15 +129,15 @@ __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const u
             mysrc[u] = s;
             const int32_t id = __shfl(my_id, s >= 0 ? s : 0);
             ids[u] = id;
-            const uint4 *row = reinterpret_cast<const uint4 *>(table + (int64_t)id * row_bytes);
+            const uint4 *row = reinterpret_cast<const uint4 *>(table + (int64_t)id * data_chunks * 16);
 #pragma unroll
             for (int i = 0; i < SCPL; ++i) {
                 const int c = lig + SLPR * i;
                 if (s >= 0 && c < data_chunks) r[u][i] = row[c];
                 else r[u][i] = make_uint4(0u, 0u, 0u, 0u);  // meets zeros of the query
             }
-            if (s >= 0 && lig == 0) tail[u] = *reinterpret_cast<const float4 *>(row + data_chunks);
-            else tail[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (s >= 0 && lig == 0) tail[u] = *reinterpret_cast<const uint2 *>(tails + (int64_t)id * kSketchTailBytes);
+            else tail[u] = make_uint2(0u, 0u);
         }
 #pragma unroll
         for (int u = 0; u < SU; ++u) {
@@ -137,7 +154,8 @@ __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const u
             // a lane's two sums are below 2^24 (at most 64 elements of 127 * 127 each), so they convert exactly
             const float acc = fold_lanes<SLPR>(__builtin_fmaf(128.0f, (float)sh, (float)sl));
             if (lig == 0 && mysrc[u] >= 0) {
-                const float scale = tail[u].x, resid = tail[u].y, norm = tail[u].z;
+                const float scale = __builtin_bit_cast(float, tail[u].x);
+                const float resid = half_bits_as_float(tail[u].y & 0xffffu), norm = half_bits_as_float(tail[u].y >> 16);
                 const float s_hat = (scale * sq.qscale) * acc;
                 // 4e-6: the integer sums are exact, the float operations that combine them (one fused
                 // multiply-add per lane, up to six adds across lanes, two products) each round by 2^-24 of at most

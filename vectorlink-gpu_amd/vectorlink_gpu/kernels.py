@@ -179,14 +179,17 @@ def knn_exact(queries: Tensor, vectors: Tensor, k: int, metric: str = "cosine") 
 
 
 def sketch_row_bytes(dim: int) -> int:
-    """Bytes of one row of the 8-bit sketch of [N, dim] vectors."""
+    """Bytes per vector in the 8-bit sketch of [N, dim] vectors: 16 * ceil(dim / 16) of data and 8 of tail."""
     return nv.check(nv.lib().vl_sketch_row_bytes(dim))
 
 
 def build_sketch(vectors: Tensor) -> Tensor:
-    """8-bit sketch of `vectors` (no counterpart in the reference): per row the
+    """8-bit sketch of `vectors` (no counterpart in the reference): per vector the
     elements rounded to 8 bits with one scale, and how far the rounding moved the
-    row, which bounds every dot product with it.  [N, sketch_row_bytes(dim)] uint8;
+    vector, which bounds every dot product with it.  One block of
+    N * sketch_row_bytes(dim) bytes, shaped [N, sketch_row_bytes(dim)] uint8 for its
+    size only: all the data rows come first, then all the tails (sketch_parts takes
+    it apart), so a slice of it is not the sketch of a slice of the vectors.
     closest_vectors(..., sketch=...) uses it to decide which candidate rows to
     fetch; no distance it returns comes from the sketch."""
     _check_f32(vectors, "vectors")
@@ -195,6 +198,20 @@ def build_sketch(vectors: Tensor) -> Tensor:
     out = torch.empty((n, sketch_row_bytes(dim)), dtype=torch.uint8, device=vectors.device)
     nv.check(nv.lib().vl_sketch_build(nv.ptr(vectors), n, dim, nv.ptr(out), nv.stream()))
     return out
+
+
+def sketch_parts(sketch: Tensor) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """The parts of a sketch from build_sketch, as views and small copies: the int8 data rows
+    [N, 16 * ceil(dim / 16)] (zeros after column dim), and per vector its scale (float32) and the two
+    bounds the tail holds as halves, on the 2-norm of what the rounding moved and on the vector's own."""
+    (n, row_bytes) = sketch.size()
+    data_bytes = row_bytes - 8
+    flat = sketch.reshape(-1)
+    data = flat[:n * data_bytes].view(torch.int8).reshape(n, data_bytes)
+    tails = flat[n * data_bytes:].reshape(n, 8)
+    scale = tails[:, :4].contiguous().view(torch.float32).reshape(n)
+    bounds = tails[:, 4:].contiguous().view(torch.float16).reshape(n, 2)
+    return (data, scale, bounds[:, 0].float(), bounds[:, 1].float())
 
 
 def sketch_bounds(queries: Tensor, sketch: Tensor, ids: Tensor) -> Tuple[Tensor, Tensor]:
