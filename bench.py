@@ -46,7 +46,7 @@ MFMA_FP32_PEAK = 157.3  # MI355X published dense fp32 matrix TFLOP/s
 # (FETCH_SIZE x 2.0 after calibration against the 1 GiB copy + WRITE_SIZE x 1.0, "roofline pass" phases);
 # NOT measured in this run.  Workloads without a recorded counter run report null.
 TRAFFIC_PER_LOOP = {
-    "mix-1m-768": [(2072185.7 * 2 + 155367.1) * 1024, (806583.7 * 2 + 61026.9) * 1024, (417181.9 * 2 + 25924.5) * 1024],
+    "mix-1m-768": [(1963460.0 * 2 + 155342.1) * 1024, (805389.5 * 2 + 61024.5) * 1024, (416887.4 * 2 + 25923.8) * 1024],
     "mix-1m-128": [(430414.2 * 2 + 25794.5) * 1024, (231365.9 * 2 + 28947.2) * 1024, (153333.9 * 2 + 20416.3) * 1024],
 }
 
