@@ -1107,6 +1107,7 @@ def test_closest_vectors_with_sketch(n, dim, beam, bqf, pv, vqf, ef, ra, cache):
     if dim >= 64:
         v[5] = v[9]            # exact duplicate rows: ties ordered by id
         v[11] *= 1.5           # a row that is not of unit length
+        v[13] *= 1e6           # ... and one longer than the sketch's tail can say (bounds of infinity: always fetched)
     c = cfg(beam_size=beam, beam_queue_factor=bqf, parallel_visit_count=pv, visit_queue_factor=vqf,
             exclude_factor=ef, speculative_readahead=ra)
     ql = beam * bqf
@@ -1171,7 +1172,8 @@ def test_sketch_bounds_hold_for_the_exact_kernel(dim):
     distance the exact kernel returns, on random pairs and on the pairs that stress the bound - a query along
     what the rounding moved (the Cauchy-Schwarz worst case, both signs), a query equal or opposite to the row,
     a query with one huge and many tiny elements (coarse steps of its own rounding), rows that are not of unit
-    length, rows of zeros, tiny rows, NaN.  And the bounds are worth something: on unit rows hi - lo stays
+    length (one longer than a half can say: its bounds are the widest), rows of zeros, tiny rows, NaN.  And the
+    bounds are worth something: on unit rows hi - lo stays
     within 2.3 x ||q|| x (what the rounding moved)."""
     say(f"sketch bounds dim={dim}")
     from vectorlink_gpu.kernels import build_sketch, gather_distances, sketch_bounds, sketch_parts
@@ -1183,6 +1185,7 @@ def test_sketch_bounds_hold_for_the_exact_kernel(dim):
     v[2] *= 6.5
     v[4] = np.float32(1e-30) * v[4]
     v[5] *= 0.01
+    v[7] *= 1e6                                                              # longer than the largest half: bounds of infinity
     sk = build_sketch(dev(v))
     (data, scale, _, _) = (host(x) for x in sketch_parts(sk))
     u = data[:, :dim].astype(np.float64)
@@ -1215,7 +1218,7 @@ def test_sketch_bounds_hold_for_the_exact_kernel(dim):
     rows = np.arange(51, nq)
     cols = np.arange(7, m)
     sub = ids[np.ix_(rows, cols)]
-    unit_rows = np.isin(sub, [1, 2, 4, 5], invert=True)
+    unit_rows = np.isin(sub, [1, 2, 4, 5, 7], invert=True)
     gap = (hi - lo)[np.ix_(rows, cols)][unit_rows]
     want = np.linalg.norm(moved[sub[unit_rows]], axis=1)
     assert np.all(gap <= 2.3 * want * 0.5 * 2 + 1e-5) and np.all(gap > 0)

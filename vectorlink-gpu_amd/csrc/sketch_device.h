@@ -161,7 +161,10 @@ __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const u
                 // multiply-add per lane, up to six adds across lanes, two products) each round by 2^-24 of at most
                 // ||q^|| ||v^||
                 const float eps = (sq.norm2 * resid + (sq.qerr + 4e-6f * sq.norm2) * (norm + resid) + sq.exactc * norm) * 1.0001f + 2e-7f;
-                const float lo = clamp_distance(s_hat + eps), hi = clamp_distance(s_hat - eps);
+                // a row with a bound of infinity (not finite, or longer than a half can say) met by a query of
+                // zeros gives 0 x infinity: no NaN leaves here for finite inputs, the widest bounds do
+                const bool known = eps == eps;
+                const float lo = known ? clamp_distance(s_hat + eps) : 0.0f, hi = known ? clamp_distance(s_hat - eps) : 1.0f;
                 out_lo[mysrc[u]] = lo;
                 out_hi[mysrc[u]] = hi;
                 if (memo_row) memo_store_bounds(memo_row, memo_shift, ids[u], lo, hi);
