@@ -16,21 +16,28 @@ After the build:
     started from are run again with the hooks ON (HIP events around the
     launches on the launch stream, fetched rows counted on the device); the
     per-loop averages are combined with the timed build's launch counts;
-  * a timed 1 GiB device copy gives the box's measured copy bandwidth;
+  * measured ceilings of the box: a 1 GiB device copy, and the library's own
+    gathered-distance kernel over a 4.3 GiB and a 120 MiB table with ids in
+    memory order and with uniformly random ids;
   * search leg: exact kNN on MFMA tiles for ground truth, then a sweep of the
-    search-queue length; QPS is reported at the shortest queue reaching
-    recall@10 >= 0.95, for the parity loop (the reference's batch-wide stop) and
-    for the per-query early exit;
+    search-queue length; QPS (median of 5 runs timed with HIP events on the
+    launch stream) is reported at the shortest queue reaching recall@10 >= 0.95,
+    for the parity loop (the reference's batch-wide stop) and for the per-query
+    early exit; `--tuned` adds a sweep over the other search settings;
   * CPU leg: the CPU oracle (a port of the reference algorithm, op for op) on
     the 4,096 x 128 workload - all cores: whole build + 256-query search;
     one thread: one 512-row batch + the search - beside the GPU on the same
     workload, and a 768-row sample of the benchmark workload itself.
-One JSON line goes to stdout.
+ONE short JSON line (under 3 KB: the headline, `roofline`, `cpu_baseline`,
+`search`, `exact_knn`) goes to stdout, last.  Everything else measured on the
+way (per-setting sweeps, per-loop tables, launch counts per phase) is written to
+the file `--detail` names, if one is given.
 """
 import argparse
 import ctypes
 import json
 import os
+import re
 import sys
 import time
 
@@ -41,14 +48,39 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E bandwidth
 MFMA_FP32_PEAK = 157.3  # MI355X published dense fp32 matrix TFLOP/s
 
-# Bytes moved past L2 per launch of the beam-search step, per optimisation-loop state, carried over from the
-# rocprofv3 --pmc runs of this same command that profiles/beam_step_kernel_<workload>_by_phase.txt records
-# (FETCH_SIZE x 2.0 after calibration against the 1 GiB copy + WRITE_SIZE x 1.0, "roofline pass" phases);
-# NOT measured in this run.  Workloads without a recorded counter run report null.
-TRAFFIC_PER_LOOP = {
-    "mix-1m-768": [(1963460.0 * 2 + 155342.1) * 1024, (805389.5 * 2 + 61024.5) * 1024, (416887.4 * 2 + 25923.8) * 1024],
-    "mix-1m-128": [(430414.2 * 2 + 25794.5) * 1024, (231365.9 * 2 + 28947.2) * 1024, (153333.9 * 2 + 20416.3) * 1024],
-}
+PROFILE_DIR = os.path.join(ROOT, "profiles")
+LINE_LIMIT = 3072       # the one JSON line on stdout stays below this many bytes
+
+
+def traffic_from_profiles(workload):
+    """Bytes moved past L2 per launch of the beam-search step, per optimisation-loop state, read from the committed
+    rocprofv3 --pmc summary of this same command (profiles/beam_step_kernel_<workload>_by_phase.txt: FETCH_SIZE and
+    WRITE_SIZE in KiB per dispatch, each scaled by what the counter reads for the 1 GiB copy).  NOT measured in this
+    run; None when no summary for the workload is committed."""
+    path = os.path.join(PROFILE_DIR, f"beam_step_kernel_{workload}_by_phase.txt")
+    if not os.path.exists(path):
+        return None, None
+    fetch_factor = write_factor = None
+    section = None
+    per_loop = {}
+    with open(path) as f:
+        for line in f:
+            if line.startswith("## FETCH_SIZE"):
+                section = "fetch"
+            elif line.startswith("## WRITE_SIZE"):
+                section = "write"
+            m = re.search(r"# calibration: .*-> factor ([0-9.]+)", line)
+            if m and section == "fetch":
+                fetch_factor = float(m.group(1))
+            elif m and section == "write":
+                write_factor = float(m.group(1))
+            m = re.match(r"roofline pass, state of loop (\d+): FETCH_SIZE ([0-9.]+), WRITE_SIZE ([0-9.]+)", line)
+            if m:
+                per_loop[int(m.group(1))] = (float(m.group(2)), float(m.group(3)))
+    if fetch_factor is None or write_factor is None or not per_loop:
+        return None, None
+    out = [(per_loop[k][0] * fetch_factor + per_loop[k][1] * write_factor) * 1024.0 for k in sorted(per_loop)]
+    return out, os.path.relpath(path, ROOT)
 
 
 def log(*a):
@@ -84,22 +116,37 @@ def step_roofline(prof, dim, batch_rows):
                 distances_served_from_cache=(1.0 - prof["evals"] / wanted) if prof["sketched"] == 0 else None)
 
 
-def measured_read_gbs(torch, dev):
-    """Bandwidth of a read-only pass (a sum) over 4 GiB of device memory, best of 5."""
-    src = torch.empty(1 << 30, dtype=torch.float32, device=dev).fill_(1.0)
-    src.sum()
-    torch.cuda.synchronize()
-    best = None
-    for _ in range(5):
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        src.sum()
-        b.record()
-        torch.cuda.synchronize()
-        ms = a.elapsed_time(b)
-        best = ms if best is None or ms < best else best
-    del src
-    return 4.0 * (1 << 30) / (best / 1e3) / 1e9
+def gather_ceilings(torch, dev, dim):
+    """The library's own gathered-distance kernel (one distance = one row of 4*dim bytes fetched, an id read, a
+    distance written) on a table far beyond the 256 MB memory-side cache (4.3 GiB) and on one inside it (120 MiB),
+    with ids in memory order and with uniformly random ids: what this box delivers to that access pattern, best of 3."""
+    from vectorlink_gpu.kernels import gather_distances
+
+    width = 64
+    out = {}
+    for (label, rows) in (("4.3GiB", int(4.3 * 2**30) // (4 * dim)), ("120MiB", 120 * 2**20 // (4 * dim))):
+        table = torch.empty((rows, dim), dtype=torch.float32, device=dev).normal_()
+        n_q = min(max(rows // width, 16384), 65536)
+        queries = table[:n_q].contiguous()
+        g = torch.Generator(device="cpu").manual_seed(5)
+        order = (torch.arange(n_q * width, dtype=torch.int64) % rows).to(torch.int32).view(n_q, width)
+        rand = torch.randint(0, rows, (n_q, width), generator=g, dtype=torch.int32)
+        for (kind, ids) in (("sequential", order.to(dev)), ("random", rand.to(dev))):
+            res = torch.empty((n_q, width), dtype=torch.float32, device=dev)
+            gather_distances(queries, table, ids, res)
+            torch.cuda.synchronize()
+            best = None
+            for _ in range(3):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                gather_distances(queries, table, ids, res)
+                b.record()
+                torch.cuda.synchronize()
+                ms = a.elapsed_time(b)
+                best = ms if best is None or ms < best else best
+            out[f"{kind}_{label}"] = n_q * width * (4.0 * dim + 12) / (best / 1e3) / 1e9
+        del table, queries
+    return out
 
 
 def measured_copy_gbs(torch, dev):
@@ -235,6 +282,79 @@ def cpu_leg(torch, dev, base_c3, cfg_c3, cpu_rows, gpu_c3_batch):
     return out
 
 
+def _r(x, digits=4):
+    """Numbers of the printed line carry a few significant digits only."""
+    if isinstance(x, float):
+        return float(f"{x:.{digits}g}")
+    return x
+
+
+def _pick(d, keys, digits=4):
+    return {k: _r(d[k], digits) for k in keys if d is not None and k in d and d[k] is not None}
+
+
+def headline(result):
+    """The ONE line for stdout, from everything a run measured: the contract's keys, `roofline`, `cpu_baseline`,
+    `search`, `exact_knn`, a few figures each - never a sweep.  Stays under LINE_LIMIT bytes whatever `result` holds."""
+    line = {k: _r(result[k], 6) for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
+                                          "higher_is_better", "scaling", "vs_baseline", "dtype", "data") if k in result}
+    line["config"] = _pick(result.get("config", {}), ("workload", "n", "dim", "degree", "build_queue", "batch_size",
+                                                      "optimization_loops", "parallel_visit_count", "prune",
+                                                      "concurrent_batches", "queries"))
+    line.update(_pick(result, ("build_seconds", "build_steps")))
+    rf = result.get("roofline")
+    if rf is not None:
+        out = {k: rf.get(k) for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")}
+        out = {k: _r(v) for k, v in out.items()}
+        out["kernel"] = "beam_step"
+        out["scope"] = "algorithmic bytes / published HBM peak; served beyond L2"
+        out.update(_pick(rf, ("avg_launch_ms", "algorithmic_bytes_per_launch", "launches_in_timed_build",
+                              "copy_gbs_measured")))
+        if rf.get("gather_gbs_measured"):
+            out["gather_gbs_measured"] = {k: _r(v, 3) for k, v in rf["gather_gbs_measured"].items()}
+        out["per_loop"] = [_pick(r, ("loop", "avg_launch_ms", "algorithmic_bytes_per_launch", "frac",
+                                     "traffic_over_algorithmic", "build_launches_of_this_loop"), 3)
+                           for r in rf.get("per_loop", [])][:4]
+        line["roofline"] = out
+    search_keys = ("seeding", "stop", "queue", "qps", "qps_min", "qps_max", "runs", "recall_at_10", "reached_0_95")
+    short_keys = ("seeding", "stop", "queue", "qps", "recall_at_10")
+    for name in ("search", "search_per_query_stop", "search_reference_seeding"):
+        if name in result:
+            line[name] = _pick(result[name], search_keys if name == "search" else short_keys)
+    sr = (result.get("search") or {}).get("roofline")
+    if sr:
+        line["search"]["iterations"] = _pick(sr["iterations"], ("launches", "avg_launch_ms", "frac"), 3)
+        line["search"]["seeding_tiles"] = _pick(sr["seeding_tiles"], ("seconds", "tflops", "frac"), 3)
+    tuned = result.get("search_tuned")
+    if tuned:
+        keys = short_keys + ("entry_points", "seed_dims", "parallel_visit_count", "speculative_readahead")
+        line["search_tuned"] = dict(settings_tried=len(tuned.get("tried", [])), best=_pick(tuned.get("best"), keys),
+                                    best_with_the_reference_stop=_pick(tuned.get("best_with_the_reference_stop"), keys))
+    if "exact_knn" in result:
+        line["exact_knn"] = _pick(result["exact_knn"], ("bound", "seconds", "tflops", "peak_tflops", "frac"))
+    cb = result.get("cpu_baseline")
+    if cb is not None:
+        out = {k: _r(cb.get(k)) for k in ("value", "unit", "cores", "kind")}
+        out["sample"] = str(cb.get("sample", ""))[:200]
+        if "all_core" in cb:
+            out["search_qps"] = _r(cb["all_core"].get("search_qps"))
+        if "gpu_same_workload" in cb:
+            out["gpu_same_workload"] = _pick(cb["gpu_same_workload"], ("build_vectors_per_s", "search_qps",
+                                                                       "graph_and_search_ids_equal_the_cpu"))
+        if "benchmark_workload_sample" in cb:
+            out["benchmark_workload_sample"] = _pick(cb["benchmark_workload_sample"],
+                                                     ("rows", "seconds", "rows_per_s_first_loop",
+                                                      "ids_and_distances_match_gpu"))
+        line["cpu_baseline"] = out
+    text = json.dumps(line)
+    if len(text) >= LINE_LIMIT:   # never happens with the keys above; if it ever does, the optional parts go first
+        for k in ("search_reference_seeding", "search_per_query_stop", "search_tuned"):
+            line.pop(k, None)
+            if len(json.dumps(line)) < LINE_LIMIT:
+                break
+    return line
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -246,7 +366,12 @@ def main():
     ap.add_argument("--n", type=int, default=None, help="override the number of vectors")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-search", action="store_true", help="skip the search leg")
-    ap.add_argument("--no-tuned", action="store_true", help="skip the sweep of search settings (search_tuned)")
+    ap.add_argument("--tuned", action="store_true",
+                    help="also sweep the other search settings (entry points, columns ranked, nodes visited per "
+                         "iteration, progress-check cadence, stop): a few hundred searches; off by default")
+    ap.add_argument("--no-tuned", action="store_true", help="accepted for older command lines; the sweep is off by default")
+    ap.add_argument("--detail", default=None,
+                    help="write everything measured (sweeps, per-loop tables, launches per phase) to this JSON file")
     ap.add_argument("--knn-only", action="store_true",
                     help="only the dense MFMA tiles on this workload's vectors (exact kNN of the queries, and the "
                          "seeding pass over 32,768 entry points); prints their figures as the JSON line")
@@ -326,8 +451,9 @@ def main():
     phases.mark("warm-up")
 
     copy_gbs = measured_copy_gbs(torch, dev)
-    read_gbs = measured_read_gbs(torch, dev)
-    log(f"[bench] 1 GiB device copy: {copy_gbs:.0f} GB/s; read-only pass over 4 GiB: {read_gbs:.0f} GB/s")
+    gather_gbs = gather_ceilings(torch, dev, dim)
+    log(f"[bench] 1 GiB device copy: {copy_gbs:.0f} GB/s; gathered distances (GB/s): "
+        + ", ".join(f"{k} {v:.0f}" for k, v in gather_gbs.items()))
 
     # ---- the timed build: whole, hooks off ----
     profile_read(nv, reset=True, enable=0)
@@ -357,7 +483,8 @@ def main():
     if t_first_k is None:
         (k_steps, t_first_k) = (done, t_build)
     value = n / t_build
-    log(f"[bench] build: {done} steps in {t_build:.1f} s -> {value:.0f} vectors/s; loops: {build.stats}")
+    log(f"[bench] build: {done} steps in {t_build:.1f} s -> {value:.0f} vectors/s; seconds per loop: "
+        + ", ".join(f"{st['seconds']:.1f}" for st in build.stats))
 
     # ---- roofline pass: the first batches of every loop's starting state again, hooks on ----
     batch_rows = min(cfg["batch_size"], n)
@@ -382,23 +509,29 @@ def main():
     w_bytes = sum(wt * r["algorithmic_bytes_per_launch"] for wt, r in zip(weights, per_loop))
     w_launch = max(sum(weights), 1)
     achieved = w_bytes / (w_time / 1e3) / 1e9 if w_time > 0 else 0.0
-    per_loop_traffic = TRAFFIC_PER_LOOP.get(args.workload)
+    (per_loop_traffic, traffic_file) = traffic_from_profiles(args.workload)
     traffic = traffic_detail = None
     if per_loop_traffic and len(per_loop_traffic) >= len(per_loop) and args.n is None:
         traffic = sum(wt * tb for wt, tb in zip(weights, per_loop_traffic)) / w_launch
+        for tb, r in zip(per_loop_traffic, per_loop):
+            r["traffic_bytes_per_launch"] = tb
+            r["traffic_over_algorithmic"] = tb / max(r["algorithmic_bytes_per_launch"], 1.0)
+            # where the counter shows fewer bytes leaving L2 than the algorithm asks for, part of them are L2 hits:
+            # the HBM-side rate is the counter's bytes over the launch time
+            r["frac_of_peak_by_counter_bytes"] = tb / (r["avg_launch_ms"] / 1e3) / 1e9 / HBM_PEAK_GBS
         traffic_detail = dict(
-            source=f"profiles/beam_step_kernel_{args.workload}_by_phase.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of "
-                   "this command, committed); not measured in this run",
-            bytes_per_launch_by_loop=per_loop_traffic[:len(per_loop)],
-            over_algorithmic_by_loop=[tb / max(r["algorithmic_bytes_per_launch"], 1.0)
-                                      for tb, r in zip(per_loop_traffic, per_loop)])
+            source=f"{traffic_file} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, committed); "
+                   "not measured in this run",
+            bytes_per_launch_by_loop=per_loop_traffic[:len(per_loop)])
     roofline = dict(
         bound="hbm",
         kernel="beam_step_kernel (one beam-search iteration: gathered cosine distances + queue merge per row)",
         achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
+        frac_scope="algorithmic bytes over the published HBM peak; the bytes are served by the path beyond L2 "
+                   "(memory-side cache + HBM), see gather_gbs_measured for what that path delivers on this box",
         traffic=traffic, traffic_detail=traffic_detail,
         copy_gbs_measured=copy_gbs, frac_of_measured_copy=achieved / copy_gbs if copy_gbs > 0 else None,
-        read_gbs_measured=read_gbs, frac_of_measured_read=achieved / read_gbs if read_gbs > 0 else None,
+        gather_gbs_measured=gather_gbs,
         avg_launch_ms=w_time / w_launch, algorithmic_bytes_per_launch=w_bytes / w_launch,
         launches_in_timed_build=int(sum(weights)),
         method=f"hooks are off in the timed build; the first {replay} batches of the tables each optimisation loop "
@@ -439,19 +572,25 @@ def main():
         flops = 2.0 * qdev.shape[0] * n * dim
         result["exact_knn"] = dict(seconds=t_knn, tflops=flops / t_knn / 1e12, peak_tflops=MFMA_FP32_PEAK,
                                    frac=flops / t_knn / 1e12 / MFMA_FP32_PEAK, bound="mfma")
-        log(f"[bench] exact kNN: {result['exact_knn']}")
+        log(f"[bench] exact kNN: {t_knn:.3f} s = {result['exact_knn']['tflops']:.1f} TFLOP/s")
 
-        def one_search(qs, seeding, mode, quiet=False):
+        def one_search(qs, seeding, mode, runs=5):
+            """Median of `runs` whole searches of all queries, each between two HIP events on the launch stream
+            (the search's own progress checks synchronise the host in between, as in any use of it)."""
             ann.search(qdev[:256].contiguous(), queue_size=qs, seeding=seeding, stop=mode)  # warm this shape
             torch.cuda.synchronize()
-            t0 = time.time()
-            res = ann.search(qdev, queue_size=qs, seeding=seeding, stop=mode)
-            torch.cuda.synchronize()
-            dt = time.time() - t0
-            r = dict(queue=qs, qps=qdev.shape[0] / dt, recall_at_10=recall_at(res.indices[:, :10], truth))
-            if not quiet:
-                log(f"[bench] search: {seeding} seeds, {mode} stop, {r}")   # a line per setting: long legs stay audible
-            return r
+            times = []
+            for _ in range(runs):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                res = ann.search(qdev, queue_size=qs, seeding=seeding, stop=mode)
+                b.record()
+                torch.cuda.synchronize()
+                times.append(a.elapsed_time(b) / 1e3)
+            times.sort()
+            nq = qdev.shape[0]
+            return dict(queue=qs, qps=nq / times[len(times) // 2], qps_min=nq / times[-1], qps_max=nq / times[0],
+                        runs=runs, recall_at_10=recall_at(res.indices[:, :10], truth))
 
         def sweep_search(seeding, mode):
             sweep, chosen = [], None
@@ -461,8 +600,9 @@ def main():
                     chosen = sweep[-1]
                     break   # the shortest queue that reaches the target is the one reported
             best = chosen or max(sweep, key=lambda r: r["recall_at_10"])
-            return dict(seeding=seeding, stop=mode, sweep=sweep, reached_0_95=chosen is not None, queue=best["queue"],
-                        qps=best["qps"], recall_at_10=best["recall_at_10"])
+            log(f"[bench] search: {seeding} seeds, {mode} stop: " + "; ".join(
+                f"queue {r['queue']} {r['qps'] / 1e3:.0f}k QPS recall {r['recall_at_10']:.4f}" for r in sweep))
+            return dict(seeding=seeding, stop=mode, sweep=sweep, reached_0_95=chosen is not None, **best)
 
         # query-dependent seeds from dense MFMA tiles over 32,768 entry points (what reaches the recall target);
         # "batch" = the reference's stop (the whole batch runs until no row changed), bit-exact against the oracle
@@ -496,7 +636,7 @@ def main():
         keep = (ann.entry_points, ann.configuration["speculative_readahead"], ann.seed_dims,
                 ann.configuration["parallel_visit_count"])
         seen_settings = set()
-        for entry_points in () if args.no_tuned else (32_768, 16_384, 8_192):
+        for entry_points in (32_768, 16_384, 8_192) if args.tuned else ():
             for seed_dims in (None, 256 if dim > 256 else None, 128 if dim > 128 else None):
                 if (entry_points, seed_dims) in seen_settings:
                     continue
@@ -508,7 +648,7 @@ def main():
                                 ann.entry_points, ann.seed_dims, ann._entry = entry_points, seed_dims, None
                                 ann.configuration["speculative_readahead"] = readahead
                                 ann.configuration["parallel_visit_count"] = visit
-                                r = one_search(qs, "dense", mode, quiet=True)
+                                r = one_search(qs, "dense", mode, runs=3)
                                 r.update(entry_points=entry_points, seed_dims=seed_dims, parallel_visit_count=visit,
                                          speculative_readahead=readahead, stop=mode)
                                 tuned.append(r)
@@ -532,12 +672,10 @@ def main():
         (ann.entry_points, ann.configuration["speculative_readahead"], ann.seed_dims,
          ann.configuration["parallel_visit_count"]) = keep
         ann._entry = None
-        result["search_tuned"] = dict(tried=tuned, **winners)
+        if args.tuned:
+            result["search_tuned"] = dict(tried=tuned, **winners)
+            log(f"[bench] search (tuned): {winners['best']}")
         phases.mark("search leg")
-        log(f"[bench] search (dense seeds): {result['search']}")
-        log(f"[bench] search (per-query stop): {result['search_per_query_stop']}")
-        log(f"[bench] search (tuned): {result['search_tuned']['best']}")
-        log(f"[bench] search (circulant seeds): {result['search_reference_seeding']}")
 
     if not args.no_cpu:
         def gpu_c3_batch(n_rows):
@@ -558,7 +696,11 @@ def main():
 
     phases.mark("CPU leg (the GPU's side of its comparisons)")
     result["beam_step_launches_by_phase"] = phases.rows
-    print(json.dumps(result), flush=True)
+    if args.detail:
+        os.makedirs(os.path.dirname(os.path.abspath(args.detail)), exist_ok=True)
+        with open(args.detail, "w") as f:
+            json.dump(result, f, indent=1)
+    print(json.dumps(headline(result)), flush=True)
 
 
 if __name__ == "__main__":
