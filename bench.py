@@ -169,16 +169,17 @@ def measured_copy_gbs(torch, dev):
 
 
 class Phases:
-    """Beam-search launches per phase of this run, in order, so that a profiler's list of
-    beam_step_kernel dispatches can be cut into the same phases."""
+    """Beam-search launches per phase of this run, in order, so that a profiler's list of beam-search step
+    dispatches (beam_step_*, beam_window_*) can be cut into the same phases."""
 
     def __init__(self):
-        from vectorlink_gpu import log as vl_log
+        from vectorlink_gpu import _native as nv
 
-        self.log, self.rows, self.last = vl_log, [], vl_log.BEAM_ITERATIONS
+        self.count = nv.lib().vl_beam_launches
+        self.rows, self.last = [], self.count()
 
     def mark(self, name):
-        now = self.log.BEAM_ITERATIONS
+        now = self.count()
         self.rows.append(dict(phase=name, beam_step_launches=now - self.last))
         self.last = now
 

@@ -22,8 +22,8 @@
  *    as a workspace whose size the matching *_workspace_bytes call reports;
  *  - threads: every entry point may be called from several host threads at
  *    once (the reference is driven from one thread).  The library's only
- *    shared state is the profiling sums of vl_beam_profile (mutex) and the
- *    thread-local error text.  A workspace belongs to ONE call at a time: the
+ *    shared state is the profiling sums of vl_beam_profile (mutex), the launch
+ *    counter of vl_beam_launches (atomic) and the thread-local error text.  A workspace belongs to ONE call at a time: the
  *    beam-search loop keeps its control block, visit queues and visited lists
  *    in it, so two vl_closest_vectors calls in flight need two workspaces;
  *  - return value 0 is success; a negative value is an error whose text
@@ -210,6 +210,15 @@ typedef struct vl_beam_params {
  * (vl_closest_vectors_with_sketch): the workspace then also holds the call's
  * query rows rounded for it (32 bytes per 16 columns and row). */
 #define VL_BEAM_USES_SKETCH 16
+/* Same loop, same result, several iterations per launch: the fused step takes
+ * a row through the speculative_readahead iterations between two progress
+ * checks in ONE launch, with the row's queues and visited list resident in LDS
+ * and a small LDS table of the (id, distance) pairs met in them, for as long as
+ * no visited list can fill up within them (parallel_visit_count * iteration <=
+ * exclude_factor * visit queue length); the stretch after that runs one
+ * iteration per launch.  Off by default (it measures slower on an MI355X: the
+ * longer kernel runs with fewer wavefronts per SIMD). */
+#define VL_BEAM_WINDOWS 32
 
 int64_t vl_beam_workspace_bytes(const vl_beam_params *p);
 
@@ -326,6 +335,12 @@ int vl_closest_vectors_noalloc(const vl_beam_params *p,
  * sketch.  The sums are kept under a mutex, so
  * profiled calls from several host threads add up without tearing. */
 int vl_beam_profile(int enable, int reset, double *out);
+
+/* Beam-search step launches (one iteration, or one window of iterations, of one
+ * batch each) enqueued by this process since the library was loaded, whatever
+ * the profiling switch says; lets a caller cut a profiler's dispatch list into
+ * the phases of its own run.  No counterpart in the reference. */
+int64_t vl_beam_launches(void);
 
 /* ---- pruning (kernels.py:441-468 prune_) ------------------------------ */
 

@@ -306,11 +306,13 @@ BEAM_CASES = [
 
 
 @pytest.mark.parametrize("n,dim,beam,bqf,pv,vqf,ef,ra", BEAM_CASES)
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", [True, False, "windows"])
 def test_closest_vectors_build_step(n, dim, beam, bqf, pv, vqf, ef, ra, fused):
+    """fused: one launch per iteration (the default); False: the loop statement by statement on the
+    single-purpose kernels; "windows": the iterations between two progress checks in one launch."""
     say(f"closest_vectors n={n} dim={dim} beam={beam} fused={fused}")
     from vectorlink_gpu import Queue
-    from vectorlink_gpu.ann import closest_vectors, closest_vectors_stepwise, excluding_self
+    from vectorlink_gpu.ann import BEAM_WINDOWS, closest_vectors, closest_vectors_stepwise, excluding_self
 
     rng = np.random.default_rng(n + dim)
     v = unit(rng, n, dim)
@@ -327,21 +329,25 @@ def test_closest_vectors_build_step(n, dim, beam, bqf, pv, vqf, ef, ra, fused):
     gv, gb = dev(v), dev(beams)
     gq = Queue(hi - lo, ql, ql + ql * pv)
     gq.insert(gb[lo:hi], dev(d)[lo:hi])
-    fn = closest_vectors if fused else closest_vectors_stepwise
-    t_got = fn(gv[lo:hi], gq, gv, gb, c, excluding_self(lo, hi))
+    if fused == "windows":
+        t_got = closest_vectors(gv[lo:hi], gq, gv, gb, c, excluding_self(lo, hi), flags=BEAM_WINDOWS)
+    else:
+        fn = closest_vectors if fused else closest_vectors_stepwise
+        t_got = fn(gv[lo:hi], gq, gv, gb, c, excluding_self(lo, hi))
     assert t_got == t_want
     assert np.array_equal(host(gq.indices)[:, :ql], oq.indices[:, :ql])
     assert np.array_equal(bits(host(gq.distances)[:, :ql]), bits(oq.distances[:, :ql]))
 
 
+@pytest.mark.parametrize("windows", [False, True])
 @pytest.mark.parametrize("ra,ef,vqf", [(5, 2, 2), (1, 1, 2), (2, 3, 1), (3, 1, 3)])
-def test_closest_vectors_many_rows_short_visited_list(ra, ef, vqf):
+def test_closest_vectors_many_rows_short_visited_list(ra, ef, vqf, windows):
     """Thousands of rows per launch with a visited list that fills up after a few iterations:
     the batch-wide state (first free column, changed flags) is read and raised by
     workgroups that are in different phases of the same launch."""
-    say(f"closest_vectors 30000 rows, readahead={ra} exclude_factor={ef}")
+    say(f"closest_vectors 30000 rows, readahead={ra} exclude_factor={ef} windows={windows}")
     from vectorlink_gpu import Queue
-    from vectorlink_gpu.ann import closest_vectors, excluding_self
+    from vectorlink_gpu.ann import BEAM_WINDOWS, closest_vectors, excluding_self
 
     rng = np.random.default_rng(77 + ra)
     n, dim, beam, bqf, pv = 30000, 8, 4, 2, 4
@@ -358,10 +364,40 @@ def test_closest_vectors_many_rows_short_visited_list(ra, ef, vqf):
     for attempt in range(3):  # the interleaving of workgroups differs from run to run
         gq = Queue(n, ql, ql + ql * pv)
         gq.insert(gb, dev(d))
-        t_got = closest_vectors(gv, gq, gv, gb, c, excluding_self(0, n))
+        t_got = closest_vectors(gv, gq, gv, gb, c, excluding_self(0, n), flags=BEAM_WINDOWS if windows else 0)
         assert t_got == t_want
         assert np.array_equal(host(gq.indices)[:, :ql], oq.indices[:, :ql])
         assert np.array_equal(bits(host(gq.distances)[:, :ql]), bits(oq.distances[:, :ql]))
+
+
+@pytest.mark.parametrize("ra", [2, 3, 5, 8])
+def test_windows_with_rows_that_start_late_in_a_launch(ra):
+    """Several iterations per launch on a batch of more workgroups than the GPU holds at once (3,500 rows
+    of 128 threads): rows that start after others of the same launch have finished must not see what those
+    wrote for the launch after it (the largest visited-list fill, whose slot is the one an iteration reads
+    for "the lists were full an iteration ago" when the launch spans 2, 5, 8, ... iterations)."""
+    say(f"windows of {ra} iterations, 3500 rows")
+    from vectorlink_gpu import Queue
+    from vectorlink_gpu.ann import BEAM_WINDOWS, closest_vectors, excluding_self
+
+    rng = np.random.default_rng(4242)
+    n, dim, beam, bqf, pv = 6000, 32, 8, 2, 4
+    v = unit(rng, n, dim)
+    c = cfg(beam_size=beam, beam_queue_factor=bqf, parallel_visit_count=pv, speculative_readahead=ra)
+    ql = beam * bqf
+    beams = orc.generate_circulant_beams(n, orc.primes(ql))
+    d = orc.calculate_distances(v, beams)
+    lo, hi = 2500, 6000
+    oq = orc.Queue(hi - lo, ql, ql + ql * pv)
+    oq.insert(beams[lo:hi], d[lo:hi])
+    t_want = orc.closest_vectors(v[lo:hi], oq, v, beams, c, orc.excluding_self(lo, hi))
+    gv, gb = dev(v), dev(beams)
+    gq = Queue(hi - lo, ql, ql + ql * pv)
+    gq.insert(gb[lo:hi], dev(d)[lo:hi])
+    t_got = closest_vectors(gv[lo:hi], gq, gv, gb, c, excluding_self(lo, hi), flags=BEAM_WINDOWS)
+    assert t_got == t_want
+    assert np.array_equal(host(gq.indices)[:, :ql], oq.indices[:, :ql])
+    assert np.array_equal(bits(host(gq.distances)[:, :ql]), bits(oq.distances[:, :ql]))
 
 
 def test_generate_ann_and_search_against_oracle():
@@ -756,13 +792,15 @@ def test_hand_enumerated_chain_on_the_gpu():
         assert host(q.indices)[0, :2].tolist() == ids_want and host(q.distances)[0, :2].tolist() == d_want
 
 
+@pytest.mark.parametrize("windows", [False, True])
 @pytest.mark.parametrize("n,dim,beam,bqf,pv,vqf,ef,ra", BEAM_CASES)
-def test_per_query_stop_against_its_model(n, dim, beam, bqf, pv, vqf, ef, ra):
+def test_per_query_stop_against_its_model(n, dim, beam, bqf, pv, vqf, ef, ra, windows):
     """VL_BEAM_PER_QUERY_STOP against the CPU model that defines it (oracle.closest_vectors_per_query):
-    same iteration count, ids and distance bits, on a build step with self exclusion."""
-    say(f"per-query stop n={n} dim={dim} beam={beam}")
+    same iteration count, ids and distance bits, on a build step with self exclusion; also with several
+    iterations per launch."""
+    say(f"per-query stop n={n} dim={dim} beam={beam} windows={windows}")
     from vectorlink_gpu import Queue
-    from vectorlink_gpu.ann import BEAM_PER_QUERY_STOP, closest_vectors, excluding_self
+    from vectorlink_gpu.ann import BEAM_PER_QUERY_STOP, BEAM_WINDOWS, closest_vectors, excluding_self
 
     rng = np.random.default_rng(1000 + n + dim)
     v = unit(rng, n, dim)
@@ -778,7 +816,8 @@ def test_per_query_stop_against_its_model(n, dim, beam, bqf, pv, vqf, ef, ra):
     gv, gb = dev(v), dev(beams)
     gq = Queue(hi - lo, ql, ql + ql * pv)
     gq.insert(gb[lo:hi], dev(d)[lo:hi])
-    t_got = closest_vectors(gv[lo:hi], gq, gv, gb, c, excluding_self(lo, hi), flags=BEAM_PER_QUERY_STOP)
+    t_got = closest_vectors(gv[lo:hi], gq, gv, gb, c, excluding_self(lo, hi),
+                            flags=BEAM_PER_QUERY_STOP | (BEAM_WINDOWS if windows else 0))
     assert t_got == t_want
     assert np.array_equal(host(gq.indices)[:, :ql], oq.indices[:, :ql])
     assert np.array_equal(bits(host(gq.distances)[:, :ql]), bits(oq.distances[:, :ql]))
@@ -1088,18 +1127,18 @@ SKETCH_CASES = [
 
 
 @pytest.mark.parametrize("n,dim,beam,bqf,pv,vqf,ef,ra", SKETCH_CASES)
-@pytest.mark.parametrize("cache", [False, True])
+@pytest.mark.parametrize("cache", [False, True, "windows"])
 def test_closest_vectors_with_sketch(n, dim, beam, bqf, pv, vqf, ef, ra, cache):
-    """The loop with the 8-bit sketch against the oracle: same iteration count, ids and distance bits.
-    Without the distance cache every row looks through the sketch from the first iteration; with it, rows
-    measure their share of cache hits first (random rows on a circulant graph: hardly any) and then switch.
-    The profiling counters show that the sketch was really used."""
+    """The loop with the 8-bit sketch against the oracle: same iteration count, ids and distance bits, without
+    the distance cache, with it (a probe then finds exact distances and bounds), and with cache, sketch and
+    several iterations per launch (the LDS table in front of the cache).  Every row starts out looking through
+    the sketch from its second iteration; the profiling counters show that it was really used."""
     say(f"closest_vectors with sketch n={n} dim={dim} beam={beam} cache={cache}")
     import ctypes
 
     from vectorlink_gpu import Queue
     from vectorlink_gpu import _native as nv
-    from vectorlink_gpu.ann import BEAM_NO_CACHE, closest_vectors, excluding_self
+    from vectorlink_gpu.ann import BEAM_NO_CACHE, BEAM_WINDOWS, closest_vectors, excluding_self
     from vectorlink_gpu.kernels import build_sketch
 
     rng = np.random.default_rng(n + dim)
@@ -1125,8 +1164,8 @@ def test_closest_vectors_with_sketch(n, dim, beam, bqf, pv, vqf, ef, ra, cache):
     out = (ctypes.c_double * 9)()
     nv.lib().vl_beam_profile(1, 1, out)
     try:
-        t_got = closest_vectors(gv[lo:hi], gq, gv, gb, c, excluding_self(lo, hi), flags=0 if cache else BEAM_NO_CACHE,
-                                sketch=sk)
+        flags = {False: BEAM_NO_CACHE, True: 0, "windows": BEAM_WINDOWS}[cache]
+        t_got = closest_vectors(gv[lo:hi], gq, gv, gb, c, excluding_self(lo, hi), flags=flags, sketch=sk)
     finally:
         nv.lib().vl_beam_profile(0, 1, out)
     (fetched, wanted, sketched) = (out[4], out[7], out[8])
@@ -1135,11 +1174,9 @@ def test_closest_vectors_with_sketch(n, dim, beam, bqf, pv, vqf, ef, ra, cache):
     assert np.array_equal(host(gq.indices)[:, :ql], oq.indices[:, :ql])
     assert np.array_equal(bits(host(gq.distances)[:, :ql]), bits(oq.distances[:, :ql]))
     if dim % 4 == 0 and dim <= 2048:
-        if not cache:
-            # every row starts with the sketch; rows that end up fetching more than half of their candidates
-            # anyway (these small iid tables put many within the sketch's error of the queues' ends) give it up
-            assert 0 < sketched <= wanted
-        # with the cache, rows switch only if few of their candidates repeat and few of them matter
+        # every row starts with the sketch; rows that end up fetching more than half of their candidates
+        # anyway (these small iid tables put many within the sketch's error of the queues' ends) give it up
+        assert 0 < sketched <= wanted
     else:
         assert sketched == 0
 

@@ -22,6 +22,7 @@
 #include "dist_device.h"
 #include "sketch_device.h"
 #include <stdlib.h>
+#include <atomic>
 #include <mutex>
 
 int vl_launch_expand(const float *queries, int64_t n_rows, const float *vectors, int64_t n_vectors,
@@ -49,6 +50,7 @@ struct BeamProfile {
 // returns, so calls on different host threads do not tear each other's sums.
 BeamProfile g_prof;
 std::mutex g_prof_mutex;
+std::atomic<int64_t> g_step_launches{0};  // vl_beam_launches
 
 // HIP events of one profiled call; destroyed on every way out of the call.
 struct EventSet {
@@ -446,19 +448,36 @@ struct NoRefine {
     __device__ __forceinline__ void operator()(const int32_t *, int, bool, uint64_t, uint64_t, uint8_t *, uint64_t *) const {}
 };
 
-template <int THREADS, bool FUSED, class Refine = NoRefine>
-__device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *smem, RowState pre = RowState{0, 0},
-                                          Refine refine = Refine()) {
+// RESIDENT (a workgroup that takes its row through several iterations, beam_window_body): the row's queues and
+// visited list stay in LDS between iterations.  The merge phase reads them where this says and writes the merged
+// queues to the *_out arrays instead of memory; nothing of the row goes to memory here.
+struct ResidentRow {
+    uint64_t *qa, *qa_out;    // search queue [0, L) as keys
+    uint64_t *va, *va_out;    // visit queue, all VL slots (the popped heads first)
+    int32_t *seen_a, *seen_b; // visited list before / after this iteration
+    int32_t *exl;
+    uint8_t *fl;
+    int *quiet;               // per-query stop: the row's count of quiet iterations
+};
+struct MergeResult {
+    int cnt;           // fill of the visited list after this iteration
+    bool queue_moved;  // RESIDENT: the search queue was written to qa_out (else it is unchanged in qa)
+};
+
+template <int THREADS, bool FUSED, class Refine = NoRefine, bool RESIDENT = false>
+__device__ __forceinline__ MergeResult merge_row(const MergeArgs &a, unsigned char *smem, RowState pre = RowState{0, 0},
+                                                 Refine refine = Refine(), const ResidentRow *rr = nullptr) {
+    static_assert(FUSED || !RESIDENT, "a resident row is a fused one");
     const int Pc = a.Pc;
     uint64_t *raw = reinterpret_cast<uint64_t *>(smem);  // candidate keys as they arrive
     uint64_t *uk = raw + Pc;                             // the candidates that can matter, then sorted
-    uint64_t *cc = uk + Pc;                              // filtered for one merge
-    uint64_t *qa = cc + Pc;                              // search queue [0, L)
-    uint64_t *va = qa + a.L;                             // visit queue [Vt, VL)
-    int32_t *seen_a = reinterpret_cast<int32_t *>(va + a.VL);
-    int32_t *seen_b = seen_a + a.E;
-    int32_t *exl = seen_b + a.E;
-    uint8_t *fl = reinterpret_cast<uint8_t *>(exl + a.excl_cols);  // per candidate: bit0 wanted, bit1 rest
+    uint64_t *cc = RESIDENT ? raw : uk + Pc;             // filtered for one merge (raw is no longer needed by then)
+    uint64_t *qa = RESIDENT ? rr->qa : cc + Pc;          // search queue [0, L)
+    uint64_t *va = RESIDENT ? rr->va + a.Vt : qa + a.L;  // visit queue [Vt, VL)
+    int32_t *seen_a = RESIDENT ? rr->seen_a : reinterpret_cast<int32_t *>(va + a.VL);
+    int32_t *seen_b = RESIDENT ? rr->seen_b : seen_a + a.E;
+    int32_t *exl = RESIDENT ? rr->exl : seen_b + a.E;
+    uint8_t *fl = RESIDENT ? rr->fl : reinterpret_cast<uint8_t *>(exl + a.excl_cols);  // per candidate: bit0 wanted, bit1 rest
     __shared__ int wave_cnt[kQueueWaves];
     __shared__ uint64_t red[2 * kQueueWaves];
     __shared__ int32_t newv[kMaxVisit];
@@ -518,11 +537,11 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
             }
         }
     }
-    if (stop) return;
+    if (stop) return MergeResult{cnt, false};
     if (!FUSED && t >= 2 && first_prev >= a.E) {
         // the visit queue is no longer fed: every candidate of this iteration is empty
         if (threadIdx.x == 0) raise_running_max(first_next, cnt, min(a.E, a.Vt * t));
-        return;
+        return MergeResult{cnt, false};
     }
     const bool seen_full = first >= a.E;
     const bool checking = (t % a.readahead) == 0;
@@ -561,13 +580,17 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
             seen_b[lower_bound(seen_a, cnt, newv[threadIdx.x]) + threadIdx.x] = newv[threadIdx.x];
         __syncthreads();
         cnt += n_new;
-        if (n_new) {
-            int32_t *srow = a.seen + row * a.E;
-            for (int i = threadIdx.x; i < cnt; i += blockDim.x) srow[i] = seen_b[i];
+        if constexpr (!RESIDENT) {
+            if (n_new) {
+                int32_t *srow = a.seen + row * a.E;
+                for (int i = threadIdx.x; i < cnt; i += blockDim.x) srow[i] = seen_b[i];
+            }
+            if (threadIdx.x == 0 && n_new) a.seen_count[row] = cnt;
         }
-        if (threadIdx.x == 0 && n_new) a.seen_count[row] = cnt;
     }
-    if (threadIdx.x == 0) raise_running_max(first_next, cnt, min(a.E, a.Vt * t));
+    if constexpr (!RESIDENT) {
+        if (threadIdx.x == 0) raise_running_max(first_next, cnt, min(a.E, a.Vt * t));
+    }
     if constexpr (FUSED) {
         refine(seen_b, cnt, seen_full, qa[a.L - 1], nva > 0 ? va[nva - 1] : 0ull, fl, red);
         // a thread packs the slots it (or a lane of its own wavefront, before the barrier above or in refine) wrote
@@ -648,7 +671,9 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
         for (int i = threadIdx.x; i < a.L; i += blockDim.x) {
             uint64_t k = qa[i];
             int r = i + key_lower_bound(cc, n_s, k);
-            if (r != i && r < a.L) {
+            if constexpr (RESIDENT) {
+                if (r < a.L) rr->qa_out[r] = k;
+            } else if (r != i && r < a.L) {
                 qi[r] = vl_key_id(k);
                 qd[r] = vl_key_dist(k);
             }
@@ -657,8 +682,12 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
             uint64_t k = cc[j];
             int r = j + key_lower_bound(qa, a.L, k);
             if (r < a.L) {
-                qi[r] = vl_key_id(k);
-                qd[r] = vl_key_dist(k);
+                if constexpr (RESIDENT) {
+                    rr->qa_out[r] = k;
+                } else {
+                    qi[r] = vl_key_id(k);
+                    qd[r] = vl_key_dist(k);
+                }
                 diff = true;  // a new id inside the first L slots: the row changed (queue.py:57-59)
             }
         }
@@ -671,9 +700,10 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
         if (diff) row_changed_s = 1;  // every writer stores the same 1
         __syncthreads();
         if (threadIdx.x == 0) {
-            int quiet = row_changed_s ? 0 : a.row_quiet[row] + 1;
+            int quiet = row_changed_s ? 0 : (RESIDENT ? *rr->quiet : a.row_quiet[row]) + 1;
             if (seen_full) quiet = a.readahead;
-            a.row_quiet[row] = quiet;
+            if constexpr (RESIDENT) *rr->quiet = quiet;
+            else a.row_quiet[row] = quiet;
             if (checking && quiet < a.readahead &&
                 __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
                 __hip_atomic_store(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -682,7 +712,7 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
         if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
             __hip_atomic_store(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (seen_full) return;
+    if (seen_full) return MergeResult{cnt, n_s > 0};
     __syncthreads();  // cc is reused below
 
     // ---- visit_queue.insert(candidates, exclude=seen) : ann.py:85-88 --------------------
@@ -699,22 +729,35 @@ __device__ __forceinline__ void merge_row(const MergeArgs &a, unsigned char *sme
         uint64_t k = va[i];
         int r = i + key_lower_bound(cc, n_v, k);
         if (r < a.VL) {
-            vi[r] = vl_key_id(k);
-            vd[r] = vl_key_dist(k);
+            if constexpr (RESIDENT) {
+                rr->va_out[r] = k;
+            } else {
+                vi[r] = vl_key_id(k);
+                vd[r] = vl_key_dist(k);
+            }
         }
     }
     for (int j = threadIdx.x; j < n_v; j += blockDim.x) {
         uint64_t k = cc[j];
         int r = j + key_lower_bound(va, nva, k);
         if (r < a.VL) {
-            vi[r] = vl_key_id(k);
-            vd[r] = vl_key_dist(k);
+            if constexpr (RESIDENT) {
+                rr->va_out[r] = k;
+            } else {
+                vi[r] = vl_key_id(k);
+                vd[r] = vl_key_dist(k);
+            }
         }
     }
     for (int r = nva + n_v + threadIdx.x; r < a.VL; r += blockDim.x) {  // the popped slots end up here, empty
-        vi[r] = VL_MAXINT;
-        vd[r] = VL_MAXFLOAT;
+        if constexpr (RESIDENT) {
+            rr->va_out[r] = vl_make_key(VL_MAXINT, VL_MAXFLOAT);
+        } else {
+            vi[r] = VL_MAXINT;
+            vd[r] = VL_MAXFLOAT;
+        }
     }
+    return MergeResult{cnt, n_s > 0};
 }
 
 template <int THREADS>
@@ -747,6 +790,8 @@ struct StepArgs {
     int sketch_chunks;         // 16-byte chunks of data in a sketch row
     const uint8_t *rounded_queries;  // the call's query rows rounded for the sketch (sketch_device.h)
     int64_t rounded_query_bytes;
+    int window;     // beam_window_kernel: iterations m.iter ... m.iter + window - 1 in this launch
+    int lds_slots;  // beam_window_kernel: entries of the row's distance table in LDS (a power of two, or 0)
 };
 
 // A probe of the distance cache is a random 8-byte read and every evaluated distance a random 8-byte
@@ -1104,6 +1149,454 @@ __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
     beam_step_body<CPL, LPR, U, GENERIC, THREADS>(s);
 }
 
+// ---- several iterations per launch ----------------------------------------------
+// While parallel_visit_count * t <= E (the visited list's width) no row's visited list can be full at
+// iteration t, so every row appends all the ids it pops (utils.py:73-75 with room for them in every row)
+// and nothing one row does in iterations t0 ... t0 + W - 1 depends on another row of the batch; the only
+// batch-wide facts, the progress flag of the checking iteration (ann.py:90-91) and the largest fill after
+// the last of them, are written once.  One workgroup then takes its row through W = speculative_readahead
+// iterations in one launch: search queue, visit queue and visited list are read once, stay in LDS (the merge
+// phase writes the merged rows to a second set of arrays, which becomes the current one) and go back to
+// memory once.  A small direct-mapped table in LDS keeps the (id, distance) or (id, bounds) entries the
+// row met in these iterations, so a repeat inside the window costs an LDS read instead of a probe of the
+// cache in memory.  Same candidates, same order, same merge code as beam_step_body: the rows are
+// bit-identical.  The launch must start right after a progress check (t0 = k * readahead + 1, W = readahead).
+template <int CPL, int LPR, int U, int THREADS, int SCPL = 0, int SLPR = 64, int SU = 1>
+__device__ __forceinline__ void beam_window_body(const StepArgs &s) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    MergeArgs a = s.m;
+    BeamCtrl *c = a.ctrl;
+    const int t0 = a.iter, W = s.window;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const int64_t row = blockIdx.x;
+    int32_t *vi = a.v_ids + row * a.VL;
+    float *vd = a.v_d + row * a.VL;
+    int32_t *qi = a.q_ids + row * a.cap;
+    float *qd = a.q_d + row * a.cap;
+    int32_t *srow = a.seen + row * a.E;
+    const int nva = a.VL - a.Vt;
+    const int seen_bound = min(a.E, a.Vt * (t0 - 1));  // the fill is at most Vt ids per earlier iteration
+    // ---- every read that depends on nothing else goes out first (as in beam_step_body)
+    const int32_t my_visit = tid < a.Vt ? vi[tid] : VL_MAXINT;
+    int cnt = a.seen_count[row];
+    const int quiet0 = a.row_quiet ? a.row_quiet[row] : 0;
+    const int memo_word0 = s.memo_rate[row];
+    int32_t pq_i[kPreQ], pv_i[kPreV], ps[kPreS];
+    float pq_d[kPreQ], pv_d[kPreV];
+#pragma unroll
+    for (int j = 0; j < kPreQ; ++j) {
+        const int i = tid + j * THREADS;
+        pq_i[j] = i < a.L ? qi[i] : VL_MAXINT;
+        pq_d[j] = i < a.L ? qd[i] : VL_MAXFLOAT;
+    }
+#pragma unroll
+    for (int j = 0; j < kPreV; ++j) {
+        const int i = tid + j * THREADS;
+        pv_i[j] = i < a.VL ? vi[i] : VL_MAXINT;
+        pv_d[j] = i < a.VL ? vd[i] : VL_MAXFLOAT;
+    }
+#pragma unroll
+    for (int j = 0; j < kPreS; ++j) {
+        const int i = tid + j * THREADS;
+        ps[j] = i < seen_bound ? srow[i] : VL_MAXINT;
+    }
+    int32_t my_excl = VL_MAXINT;
+    if (a.excl && tid < a.excl_cols) my_excl = a.excl[row * a.excl_cols + tid];
+
+    // (the visited lists cannot be full in these iterations; the slots of `first` are not read here, because rows
+    // of this very launch that finish early write the one the next launch reads)
+    const int gate = beam_gate(c, t0, a.readahead, a.E, blockIdx.x == 0 && tid == 0, false);
+    if (gate == 2) return;
+    int *first_after = &c->first[(t0 + W) % 3];  // what the launch of iteration t0 + W reads
+    const int bound_after = min(a.E, a.Vt * (t0 + W - 1));
+    if (a.row_quiet && quiet0 >= a.readahead) {
+        // this row has stopped on its own: nothing changes, only the running maximum is kept current
+        if (tid == 0) raise_running_max(first_after, cnt, bound_after);
+        return;
+    }
+    const int Pc = a.Pc;
+    uint64_t *raw = reinterpret_cast<uint64_t *>(smem);
+    uint64_t *uk = raw + Pc;
+    // two copies of each queue and of the visited list, the second right behind the first
+    uint64_t *const q0 = uk + Pc;
+    uint64_t *const v0 = q0 + 2 * a.L;
+    auto qbuf = [&](int k) -> uint64_t * { return q0 + k * a.L; };
+    auto vbuf = [&](int k) -> uint64_t * { return v0 + k * a.VL; };
+    LdsMemo lds;
+    lds.tab = s.lds_slots > 0 ? v0 + 2 * a.VL : nullptr;
+    lds.shift = 32 - (31 - __builtin_clz(s.lds_slots > 0 ? s.lds_slots : 1));
+    int32_t *const s0 = reinterpret_cast<int32_t *>(v0 + 2 * a.VL + s.lds_slots);
+    auto sbuf = [&](int k) -> int32_t * { return s0 + k * a.E; };
+    int32_t *exl = s0 + 2 * a.E;
+    const float *const q_row0 = s.queries + row * s.dim;
+    const uint8_t *const rounded_row0 = s.rounded_queries + row * s.rounded_query_bytes;
+    uint64_t *const memo_table = s.memo ? s.memo + ((uint64_t)row << (32 - s.memo_shift)) : nullptr;
+    __shared__ int probe_hits_s, probe_asked_s, quiet_s, memo_word_s;
+    int cur_q = 0, cur_v = 0, cur_s = 0;
+    bool queue_dirty = false;
+
+    // candidate id of slot c0 + lane: the neighbour list of a visited node
+    auto resolve = [&](int c0) -> int32_t {
+        const int slot = c0 + lane;
+        int32_t id = VL_MAXINT;
+        if (slot < a.m) {
+            int sidx = s.width == 1 ? slot : (int)__umulhi((uint32_t)slot, s.width_magic), k = slot - sidx * s.width;
+            int32_t node = g_visit_s[sidx];
+            if (node != VL_MAXINT && (uint32_t)node < (uint64_t)s.n_vectors) id = s.beams[(int64_t)node * s.width + k];
+        }
+        return id;
+    };
+    if (tid < a.Vt) g_visit_s[tid] = my_visit;
+    if (tid == 0) {
+        g_n_ex_s = a.excl ? a.excl_cols : 0;
+        quiet_s = quiet0;
+        memo_word_s = memo_word0;
+        probe_hits_s = 0;
+        probe_asked_s = 0;
+    }
+    __syncthreads();
+    int32_t id = resolve(wave * kWave);
+    {
+        // the row's state, read at the top, goes to LDS while the first neighbour lists are on their way
+#pragma unroll
+        for (int j = 0; j < kPreQ; ++j) {
+            const int i = tid + j * THREADS;
+            if (i < a.L) qbuf(0)[i] = vl_make_key(pq_i[j], pq_d[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < kPreV; ++j) {
+            const int i = tid + j * THREADS;
+            if (i < a.VL) vbuf(0)[i] = vl_make_key(pv_i[j], pv_d[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < kPreS; ++j) {
+            const int i = tid + j * THREADS;
+            if (i < seen_bound) sbuf(0)[i] = ps[j];
+        }
+        if (a.excl && tid < a.excl_cols) {
+            exl[tid] = my_excl;
+            if (my_excl == VL_MAXINT) atomicMin(&g_n_ex_s, tid);
+        }
+        for (int i = tid + kPreQ * THREADS; i < a.L; i += THREADS) qbuf(0)[i] = vl_make_key(qi[i], qd[i]);
+        for (int i = tid + kPreV * THREADS; i < a.VL; i += THREADS) vbuf(0)[i] = vl_make_key(vi[i], vd[i]);
+        for (int i = tid + kPreS * THREADS; i < seen_bound; i += THREADS) sbuf(0)[i] = srow[i];
+        for (int i = tid + THREADS; i < a.excl_cols; i += THREADS) {
+            int32_t e = a.excl[row * a.excl_cols + i];
+            exl[i] = e;
+            if (e == VL_MAXINT) atomicMin(&g_n_ex_s, i);
+        }
+        for (int i = tid; i < s.lds_slots; i += THREADS) lds.tab[i] = (uint64_t)(uint32_t)VL_MAXINT;  // no probe asks for it
+        __syncthreads();  // the table is probed below
+    }
+
+    for (int w = 0; w < W; ++w) {
+        const int t = t0 + w;
+        a.iter = t;
+        // The LDS addresses of an iteration are formed again from an offset the compiler cannot see through
+        // (always 0): hoisted out of this loop, the per-thread addresses of every array below would occupy some
+        // thirty registers through all of it, and cost a wavefront per SIMD.
+        int z = 0;
+        asm volatile("" : "+s"(z));
+        unsigned char *const base = smem + z;
+        uint64_t *const raw = reinterpret_cast<uint64_t *>(base);
+        uint64_t *const uk = raw + Pc;
+        uint64_t *const q0 = uk + Pc;
+        uint64_t *const v0 = q0 + 2 * a.L;
+        auto qbuf = [&](int k) -> uint64_t * { return q0 + k * a.L; };
+        auto vbuf = [&](int k) -> uint64_t * { return v0 + k * a.VL; };
+        LdsMemo lds;
+        lds.tab = s.lds_slots > 0 ? v0 + 2 * a.VL : nullptr;
+        lds.shift = 32 - (31 - __builtin_clz(s.lds_slots > 0 ? s.lds_slots : 1));
+        int32_t *const s0 = reinterpret_cast<int32_t *>(v0 + 2 * a.VL + s.lds_slots);
+        auto sbuf = [&](int k) -> int32_t * { return s0 + k * a.E; };
+        int32_t *const exl = s0 + 2 * a.E;
+        uint8_t *const xf = reinterpret_cast<uint8_t *>(exl + a.excl_cols);  // the merge phase's per-candidate flags; 16 = exact
+        int32_t *const li = reinterpret_cast<int32_t *>(uk);                 // candidate ids, distances behind them
+        float *const ld = reinterpret_cast<float *>(li + a.m);
+        float *const le = reinterpret_cast<float *>(raw);                    // upper bounds (raw is filled in the merge phase)
+        if (w > 0) {
+            if (tid < a.Vt) g_visit_s[tid] = vl_key_id(vbuf(cur_v)[tid]);  // queue.py:87-95: the heads are popped
+            if (tid == 0) {
+                probe_hits_s = 0;
+                probe_asked_s = 0;
+            }
+            __syncthreads();
+            id = resolve(wave * kWave);
+        }
+        // The query row (and its rounded form) is read again in every iteration, as a launch per iteration
+        // does: loaded once before the loop it would hold some forty registers through all of it, merge
+        // phases included.  The empty asm hides from the compiler that the address is the same each time.
+        const float *q_row = q_row0;
+        const uint8_t *rounded_row = rounded_row0;
+        asm volatile("" : "+s"(q_row), "+s"(rounded_row));
+        const int memo_word = memo_word_s;
+        const int memo_rate = memo_word & 0xffff;
+        uint64_t *memo_row = memo_table;
+        const bool resample = memo_row && t == kMemoDecide;
+        if (memo_row && memo_rate < s.memo_min_rate) memo_row = nullptr;
+        bool sketching = false;
+        if constexpr (SCPL > 0) sketching = s.sketch != nullptr && (memo_word >> 16) != 0 && t > 1;
+        const bool probing = memo_row != nullptr;
+
+        // ---- expand: ann.py:69-73 ----
+        int n_wanted = 0, n_fetched = 0, n_sketched = 0;  // counts of this wavefront
+        // A candidate the row met before comes back from the LDS table or, failing that, from the cache in
+        // memory: with its distance, or (rows that use the sketch) with its bounds.  Returns the entry or 0.
+        auto probe = [&](int32_t cid, bool bounds_too) -> uint64_t {
+            uint64_t e = 0;
+            bool hit = false;
+            if (lds.tab) {
+                e = lds_memo_load(lds, cid);
+                hit = (int32_t)((uint32_t)e & (bounds_too ? ~kMemoBounds : ~0u)) == cid;
+            }
+            if (!hit && probing) {
+                e = memo_load(memo_row, s.memo_shift, cid);
+                hit = (int32_t)((uint32_t)e & (bounds_too ? ~kMemoBounds : ~0u)) == cid;
+                if (hit && lds.tab) lds_memo_store(lds, cid, e);
+            }
+            return hit ? e : 0ull;
+        };
+        if constexpr (SCPL > 0) {
+            if (sketching) {
+                SketchQuery<SCPL> sq;
+                sketch_query_load<SCPL, SLPR>(sq, rounded_row, s.sketch_chunks);
+                for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
+                    if (c0 != wave * kWave) id = resolve(c0);
+                    const int slot = c0 + lane;
+                    const bool has = slot < a.m;
+                    bool ok = has && id != VL_MAXINT && id >= 0 && (int64_t)id < s.n_vectors;
+                    if (has) {
+                        li[slot] = ok ? id : VL_MAXINT;
+                        if (!ok) ld[slot] = VL_MAXFLOAT;
+                        xf[slot] = 0;
+                    }
+                    if (s.count_evals || resample) n_wanted += __popcll(__ballot(ok));
+                    if (ok) {
+                        const uint64_t e = probe(id, true);
+                        if (e) {  // (id 0 at distance 0 is the one entry that is all zeros: it reads as a miss and is evaluated again)
+                            if ((uint32_t)e & kMemoBounds) {
+                                ld[slot] = memo_bound_lo(e);
+                                le[slot] = memo_bound_hi(e);
+                            } else {
+                                const float d = __builtin_bit_cast(float, (uint32_t)(e >> 32));
+                                ld[slot] = d;
+                                le[slot] = d;
+                                xf[slot] = 16;  // exact already
+                            }
+                            ok = false;
+                        }
+                    }
+                    if (s.count_evals || resample) n_sketched += __popcll(__ballot(ok));
+                    wave_sketch<SCPL, SLPR, SU>(sq, s.sketch, s.sketch_tails, s.sketch_chunks, id, ok, ld + c0, le + c0,
+                                                memo_row, s.memo_shift, lds);
+                }
+                n_fetched = n_sketched;  // for the share of cache hits: what the cache did not answer
+            }
+        }
+        for (int c0 = wave * kWave; c0 < a.m && !sketching; c0 += THREADS) {
+            if (c0 != wave * kWave) id = resolve(c0);
+            const int slot = c0 + lane;
+            const bool has = slot < a.m;
+            bool ok = has && id != VL_MAXINT && id >= 0 && (int64_t)id < s.n_vectors;
+            if (has) {
+                li[slot] = ok ? id : VL_MAXINT;
+                if (!ok) ld[slot] = VL_MAXFLOAT;
+            }
+            if (s.count_evals || resample) n_wanted += __popcll(__ballot(ok));
+            if (ok) {
+                const uint64_t e = probe(id, false);
+                if (e) {
+                    ld[slot] = __builtin_bit_cast(float, (uint32_t)(e >> 32));
+                    ok = false;
+                }
+            }
+            if (s.count_evals || resample) n_fetched += __popcll(__ballot(ok));
+            wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, id, ok, ld + c0, memo_row, s.memo_shift,
+                                        s.l2 != 0, lds);
+        }
+        if (s.count_evals && lane == 0) {
+            const int stripe = (int)((blockIdx.x * (THREADS / kWave) + wave) & (kBeamStripes - 1));
+            if (n_wanted) atomicAdd(&c->wanted[stripe], (unsigned long long)n_wanted);
+            if (n_fetched && !sketching) atomicAdd(&c->evals[stripe], (unsigned long long)n_fetched);
+            if (n_sketched) atomicAdd(&c->sketched[stripe], (unsigned long long)n_sketched);
+        }
+        if (resample && lane == 0) {
+            atomicAdd(&probe_asked_s, n_wanted);
+            atomicAdd(&probe_hits_s, n_wanted - n_fetched);
+        }
+        __syncthreads();
+        if (resample && tid == 0) {
+            const int word = (probe_asked_s > 0 ? (probe_hits_s * 256) / probe_asked_s : 256) | (memo_word & (1 << 16));
+            s.memo_rate[row] = word;
+            memo_word_s = word;
+        }
+        // ---- merge: ann.py:75-88 ----
+        ResidentRow rr;
+        rr.qa = qbuf(cur_q); rr.qa_out = qbuf(cur_q ^ 1);
+        rr.va = vbuf(cur_v); rr.va_out = vbuf(cur_v ^ 1);
+        rr.seen_a = sbuf(cur_s); rr.seen_b = sbuf(cur_s ^ 1);
+        rr.exl = exl; rr.fl = xf; rr.quiet = &quiet_s;
+        const RowState pre{cnt, a.Vt * (t - 1)};  // every row has room for the Vt ids it pops (Vt * t <= E)
+        MergeResult mr;
+        if constexpr (SCPL > 0) {
+            // the same rule as beam_step_body's refine (see there), with the row's LDS table kept current
+            auto refine = [&](const int32_t *seen_b, int cnt_now, bool seen_full, uint64_t ws, uint64_t wv, uint8_t *flags,
+                              uint64_t *red) {
+                if (!sketching) return;  // uniform over the workgroup
+                const float ws_d = vl_key_dist(ws);
+                const float wv_d = nva > 0 ? vl_key_dist(wv) : -1.0f;
+                for (int i = tid; i < a.m; i += THREADS) {
+                    const int32_t cid = li[i];
+                    uint8_t f = flags[i] & 16;
+                    if (cid != VL_MAXINT) {
+                        const float lo = ld[i];
+                        bool need = !(lo > ws_d);
+                        if (!seen_full && !sorted_contains(seen_b, cnt_now, cid)) {
+                            if (!(lo > wv_d)) need = true;
+                            else f |= 2;
+                        }
+                        if (need) f |= 4;
+                    }
+                    flags[i] = f;
+                }
+                bool all_rest = false;
+                if (!seen_full) {
+                    for (int r = 0; r < a.Vt; ++r) {
+                        uint64_t mine = kPadKey;
+                        for (int i = tid; i < a.m; i += THREADS) {
+                            if ((flags[i] & (2 | 8)) != 2) continue;
+                            const uint64_t k = vl_make_key(li[i], le[i]);
+                            if (k < mine) mine = k;
+                        }
+                        const uint64_t mn = block_min_key(mine, red, r);
+                        if (mn == kPadKey) {
+                            all_rest = true;
+                            break;
+                        }
+                        const int32_t chosen = vl_key_id(mn);
+                        for (int i = tid; i < a.m; i += THREADS)
+                            if ((flags[i] & 2) && li[i] == chosen) flags[i] |= 8;
+                    }
+                }
+                int n_exact = 0, n_real = 0;
+                for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
+                    const int slot = c0 + lane;
+                    const bool has = slot < a.m;
+                    const int32_t cid = has ? li[slot] : VL_MAXINT;
+                    const uint8_t f = has ? flags[slot] : 0;
+                    const bool ok = ((f & (4 | 8)) || (all_rest && (f & 2))) && !(f & 16);
+                    if (ok) flags[slot] = f | 16;
+                    n_exact += __popcll(__ballot(ok));
+                    n_real += __popcll(__ballot(cid != VL_MAXINT && !(f & 16)));
+                    wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0, memo_row, s.memo_shift,
+                                                false, lds);
+                }
+                __syncthreads();
+                float tv = -1.0f;
+                if (!seen_full && !all_rest) {
+                    uint64_t mine = kPadKey;
+                    for (int i = tid; i < a.m; i += THREADS)
+                        if (flags[i] & 8) {
+                            const uint64_t k = ~(uint64_t)vl_float_key(ld[i]);
+                            mine = k < mine ? k : mine;
+                        }
+                    const uint64_t mn = block_min_key(mine, red, a.Vt);
+                    tv = mn == kPadKey ? -1.0f : vl_key_float((uint32_t)~mn);
+                }
+                for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
+                    const int slot = c0 + lane;
+                    const bool has = slot < a.m;
+                    const int32_t cid = has ? li[slot] : VL_MAXINT;
+                    const uint8_t f = has ? flags[slot] : 0;
+                    const bool ok = (f & 2) && !(f & 16) && !(ld[slot] > tv);
+                    if (has && cid != VL_MAXINT && !ok && !(f & 16)) {
+                        li[slot] = VL_MAXINT;
+                        ld[slot] = VL_MAXFLOAT;
+                    }
+                    n_exact += __popcll(__ballot(ok));
+                    wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0, memo_row, s.memo_shift,
+                                                false, lds);
+                }
+                if (s.count_evals && lane == 0 && n_exact)
+                    atomicAdd(&c->evals[(int)((blockIdx.x * (THREADS / kWave) + wave) & (kBeamStripes - 1))],
+                              (unsigned long long)n_exact);
+                if (t > 2 && !resample) {
+                    if (lane == 0) {
+                        atomicAdd(&probe_asked_s, n_real);
+                        atomicAdd(&probe_hits_s, n_exact);
+                    }
+                    __syncthreads();
+                    const bool quit = t > kMemoDecide ? 2 * probe_hits_s > probe_asked_s : 8 * probe_hits_s > 7 * probe_asked_s;
+                    if (tid == 0 && quit) {
+                        s.memo_rate[row] = memo_rate;
+                        memo_word_s = memo_rate;
+                        atomicAdd(&c->sketch_rows, -1);
+                    }
+                } else {
+                    __syncthreads();
+                }
+            };
+            mr = merge_row<THREADS, true, decltype(refine), true>(a, base, pre, refine, &rr);
+        } else {
+            mr = merge_row<THREADS, true, NoRefine, true>(a, base, pre, NoRefine(), &rr);
+        }
+        cnt = mr.cnt;
+        if (mr.queue_moved) {
+            cur_q ^= 1;
+            queue_dirty = true;
+        }
+        cur_v ^= 1;
+        cur_s ^= 1;
+        __syncthreads();  // the merged rows are read below and by the next iteration
+        if (a.row_quiet && quiet_s >= a.readahead) break;  // the row has stopped on its own (uniform)
+    }
+    // ---- the row goes back to memory once ----
+    // (addresses formed afresh: kept from the loads at the top they would sit in registers, or in scratch memory,
+    // through the whole loop)
+    asm volatile("" : "+s"(qi), "+s"(qd), "+s"(vi), "+s"(vd), "+s"(srow));
+    if (queue_dirty) {
+        const uint64_t *qf = qbuf(cur_q);
+        for (int i = tid; i < a.L; i += THREADS) {
+            const uint64_t k = qf[i];
+            qi[i] = vl_key_id(k);
+            qd[i] = vl_key_dist(k);
+        }
+    }
+    {
+        const uint64_t *vf = vbuf(cur_v);
+        for (int i = tid; i < a.VL; i += THREADS) {
+            const uint64_t k = vf[i];
+            vi[i] = vl_key_id(k);
+            vd[i] = vl_key_dist(k);
+        }
+        const int32_t *sf = sbuf(cur_s);
+        for (int i = tid; i < cnt; i += THREADS) srow[i] = sf[i];
+    }
+    if (tid == 0) {
+        a.seen_count[row] = cnt;
+        if (a.row_quiet) a.row_quiet[row] = quiet_s;
+        raise_running_max(first_after, cnt, bound_after);
+    }
+}
+
+// WPE: wavefronts per SIMD asked of the compiler.  The row's phases each wait on memory, so a launch is as fast
+// as it has wavefronts to switch to: the registers are capped at what the one-iteration kernel of the same shape
+// uses, and what the longer body holds beyond that (addresses for the write-back at the end, mostly) lives in
+// scratch memory, stored once and read back rarely.
+template <int CPL, int LPR, int U, int THREADS, int WPE>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPE)))
+void beam_window_kernel(StepArgs s) {
+    beam_window_body<CPL, LPR, U, THREADS>(s);
+}
+
+template <int CPL, int LPR, int U, int THREADS, int SCPL, int SLPR, int SU, int WPE>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPE)))
+void beam_window_sketch_kernel(StepArgs s) {
+    beam_window_body<CPL, LPR, U, THREADS, SCPL, SLPR, SU>(s);
+}
+
 // The same step for rows that may use the sketch.  WPE: wavefronts per SIMD the compiler is asked to leave room
 // for.  The sketch's copy of the query row takes 16 registers per chunk and lane, and a row's phases (sketch
 // pass, two rounds of exact rows, merge) each wait on memory, so residency is worth a few spilled registers:
@@ -1115,11 +1608,36 @@ void beam_step_sketch_kernel(StepArgs s) {
     beam_step_body<CPL, LPR, U, false, THREADS, SCPL, SLPR, SU>(s);
 }
 
-template <int CPL, int LPR, int U, bool GENERIC, int SCPL = 0, int SLPR = 64, int SU = 1, int WPE = 4, int UX = U>
+template <int CPL, int LPR, int U, bool GENERIC, int SCPL = 0, int SLPR = 64, int SU = 1, int WPE = 4, int UX = U,
+          int WPW = WPE>
 void launch_step(const StepArgs &s, int threads, size_t smem, hipStream_t st) {
     dim3 grid((unsigned)s.m.n_rows);
     if constexpr (SCPL > 0) {
-        if (!s.sketch) return launch_step<CPL, LPR, U, GENERIC>(s, threads, smem, st);
+        if (!s.sketch) return launch_step<CPL, LPR, U, GENERIC, 0, 64, 1, WPE, U, WPW>(s, threads, smem, st);
+    }
+    if constexpr (!GENERIC) {
+        if (s.window > 0) {  // several iterations in this launch (smem is the window kernel's size)
+            if constexpr (SCPL > 0) {
+                if (threads == 128) {
+                    auto kernel = beam_window_sketch_kernel<CPL, LPR, UX, 128, SCPL, SLPR, SU, WPW>;
+                    if (vl_allow_lds(kernel, smem) != hipSuccess) return;  // seen by the launch check
+                    hipLaunchKernelGGL(kernel, grid, dim3(128), smem, st, s);
+                } else {
+                    auto kernel = beam_window_sketch_kernel<CPL, LPR, UX, 256, SCPL, SLPR, SU, WPW>;
+                    if (vl_allow_lds(kernel, smem) != hipSuccess) return;
+                    hipLaunchKernelGGL(kernel, grid, dim3(256), smem, st, s);
+                }
+            } else if (threads == 128) {
+                auto kernel = beam_window_kernel<CPL, LPR, U, 128, WPW>;
+                if (vl_allow_lds(kernel, smem) != hipSuccess) return;
+                hipLaunchKernelGGL(kernel, grid, dim3(128), smem, st, s);
+            } else {
+                auto kernel = beam_window_kernel<CPL, LPR, U, 256, WPW>;
+                if (vl_allow_lds(kernel, smem) != hipSuccess) return;
+                hipLaunchKernelGGL(kernel, grid, dim3(256), smem, st, s);
+            }
+            return;
+        }
     }
     if constexpr (SCPL > 0) {
         if (threads == 128) {
@@ -1153,27 +1671,29 @@ int dist_variant() {
 }
 
 // The numbers after `false` are the sketch's lane shape for rows of that size (chunks per lane, lanes per row,
-// loads in flight), the wavefronts per SIMD asked for and, where given, the whole rows in flight in the sketch
-// kernel (it fetches few of them, so fewer in flight cost nothing and leave registers for another wavefront:
-// 0.40 -> 0.36 ms per launch at 384 columns): a sketch row has a quarter of the chunks, so a quarter of the
-// lanes (or of the chunks per lane) covers it.
+// loads in flight), the wavefronts per SIMD asked for, the whole rows in flight in the sketch kernel (it fetches
+// few of them, so fewer in flight cost nothing and leave registers for another wavefront: 0.40 -> 0.36 ms per
+// launch at 384 columns) and, where given, the wavefronts per SIMD asked for in the kernels that run several
+// iterations per launch.  A sketch row has a quarter of the chunks, so a quarter of the lanes (or of the chunks
+// per lane) covers it.
 int launch_step_by_dim(const StepArgs &s, bool aligned, int threads, size_t smem, hipStream_t st) {
     const int nchunks = s.nchunks;
     const int variant = dist_variant();
     if (!aligned || nchunks > 512) launch_step<1, 64, 1, true>(s, threads, smem, st);
-    else if (nchunks <= 16) launch_step<1, 16, 8, false, 1, 8, 4, 5>(s, threads, smem, st);
+    else if (nchunks <= 16) launch_step<1, 16, 8, false, 1, 8, 4, 5, 8, 6>(s, threads, smem, st);
     else if (nchunks <= 32 && variant == 1) launch_step<1, 32, 8, false>(s, threads, smem, st);
-    else if (nchunks <= 32) launch_step<2, 16, 4, false, 1, 8, 4, 5>(s, threads, smem, st);
-    else if (nchunks <= 64) launch_step<1, 64, 8, false, 2, 8, 2, 5>(s, threads, smem, st);
+    else if (nchunks <= 32) launch_step<2, 16, 4, false, 1, 8, 4, 5, 4, 6>(s, threads, smem, st);
+    else if (nchunks <= 64) launch_step<1, 64, 8, false, 2, 8, 2, 5, 8, 6>(s, threads, smem, st);
     else if (nchunks <= 96 && variant != 1) launch_step<3, 32, 4, false, 3, 8, 2, 6, 2>(s, threads, smem, st);
     else if (nchunks <= 128) launch_step<2, 64, 8, false, 2, 16, 2, 6, 2>(s, threads, smem, st);
-    else if (nchunks <= 192) launch_step<3, 64, 4, false, 3, 16, 2, 5>(s, threads, smem, st);
+    else if (nchunks <= 192) launch_step<3, 64, 4, false, 3, 16, 2, 5, 4, 6>(s, threads, smem, st);
     else if (nchunks <= 256) launch_step<4, 64, 4, false, 4, 16, 2, 5, 2>(s, threads, smem, st);
     else if (nchunks <= 320) launch_step<5, 64, 2, false, 3, 32, 2, 6, 1>(s, threads, smem, st);
     else if (nchunks <= 384) launch_step<6, 64, 2, false, 3, 32, 2, 6, 1>(s, threads, smem, st);
     else if (nchunks <= 448) launch_step<7, 64, 2, false, 4, 32, 2, 5, 1>(s, threads, smem, st);
     else launch_step<8, 64, 2, false, 4, 32, 2, 5, 1>(s, threads, smem, st);
     VL_LAUNCH_CHECK("beam_step_kernel");
+    g_step_launches.fetch_add(1, std::memory_order_relaxed);
     return VL_OK;
 }
 
@@ -1376,6 +1896,8 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     step.rounded_query_bytes = sketch_query_bytes(p->dim);
     step.sketch_tails = sketch ? sketch + sketch_tails_offset(p->n_vectors, p->dim) : nullptr;
     step.sketch_chunks = (int)sketch_data_chunks(p->dim);
+    step.window = 0;
+    step.lds_slots = 0;
     step.memo_shift = 32;
     if (step.memo) {
         int lg = 0;
@@ -1405,14 +1927,42 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     }
 
     const int R = (int)p->speculative_readahead;
+    // Several iterations per launch (beam_window_body; VL_BEAM_WINDOWS in flags, or VL_BEAM_WINDOW=1 in the
+    // environment): the R iterations between two progress checks run in one launch while no visited list can fill
+    // up in them, i.e. while Vt * (last iteration) <= E; the stretch after that runs one iteration per launch.
+    // Off by default: the longer kernel body needs some fifty registers more than the one-iteration kernel, and what
+    // it saves (one read and one write of the row's queues per iteration, four launches in five) is less than what
+    // the spilled registers or the lost wavefront per SIMD cost (measured at 1M x 768: 0.61 ms per iteration either
+    // way on the first optimisation loop's state, 0.48 instead of 0.42 ms on the second's).
+    static const bool window_env = [] {
+        const char *e = getenv("VL_BEAM_WINDOW");
+        return e && e[0] == '1';
+    }();
+    // entries of the row's distance table in LDS: room for the candidates of one iteration, 256 to 1024
+    static const int lds_slots_env = [] {
+        const char *e = getenv("VL_BEAM_LDS_SLOTS");
+        return e ? atoi(e) : -1;
+    }();
+    int lds_slots = a.Pc < 256 ? 256 : (a.Pc > 1024 ? 1024 : a.Pc);
+    if (lds_slots_env >= 0) lds_slots = lds_slots_env ? vl_next_pow2(lds_slots_env) : 0;
+    const size_t smem_window = (size_t)a.Pc * 16 + (size_t)(a.L + a.VL) * 16 + (size_t)lds_slots * 8 + (size_t)a.E * 8 +
+                               (size_t)a.excl_cols * 4 + (size_t)a.m + 16;
+    const bool use_window = use_fused && (window_env || (p->flags & VL_BEAM_WINDOWS)) && R >= 2 && aligned &&
+                            step.nchunks <= 512 && smem_window + 2048 <= kLdsPerCu;
+    auto window_fits = [&](int64_t first_iteration) { return use_window && l.Vt * (first_iteration + R - 1) <= l.E; };
+    const int step_threads = merge_threads == 128 ? 128 : 256;
     if (fixed_iterations > 0) {
         VL_REQUIRE(use_fused, "a fixed number of iterations is only built for the fused step");
-        for (int64_t t = 1; t <= fixed_iterations; ++t) {
+        step.count_evals = 0;
+        for (int64_t t = 1; t <= fixed_iterations;) {
             a.iter = (int)t;
             step.m = a;
-            step.count_evals = 0;
-            rc = launch_step_by_dim(step, aligned, merge_threads == 128 ? 128 : 256, smem, st);
+            const bool windowed = window_fits(t) && (t - 1) % R == 0 && t + R - 1 <= fixed_iterations;
+            step.window = windowed ? R : 0;
+            step.lds_slots = windowed ? lds_slots : 0;
+            rc = launch_step_by_dim(step, aligned, step_threads, windowed ? smem_window : smem, st);
             if (rc < 0) return rc;
+            t += windowed ? R : 1;
         }
         hipLaunchKernelGGL(beam_status_kernel, dim3(1), dim3(64), 0, st, ctrl, (int)fixed_iterations, R, status_out);
         VL_LAUNCH_CHECK("beam_status_kernel");
@@ -1444,14 +1994,31 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     int sketch_rows = sketch_from_start ? (int)p->n_rows : 0;
     int64_t t = 0;
     for (;;) {
-        for (int r = 0; r < R; ++r) {
+        int launches = 0;  // of this stretch between two progress checks
+        if (window_fits(t + 1)) {
+            // the sketch kernel also for the first window: its rows leave the sketch alone in iteration 1
+            if (prof) VL_HIP(hipEventRecord(ev[0], st));
+            a.iter = (int)(t + 1);
+            step.m = a;
+            step.sketch = (2 * (int64_t)sketch_rows >= p->n_rows) ? sketch_table : nullptr;
+            step.window = R;
+            step.lds_slots = lds_slots;
+            rc = launch_step_by_dim(step, aligned, step_threads, smem_window, st);
+            if (rc < 0) return rc;
+            if (prof) VL_HIP(hipEventRecord(ev[1], st));
+            step.window = 0;
+            step.lds_slots = 0;
+            t += R;
+            launches = 1;
+        }
+        for (int r = 0; r < R && !launches; ++r) {
             ++t;
             if (prof) VL_HIP(hipEventRecord(ev[3 * r], st));
             a.iter = (int)t;
             if (use_fused) {
                 step.m = a;
                 step.sketch = (t > 1 && 2 * (int64_t)sketch_rows >= p->n_rows) ? sketch_table : nullptr;
-                rc = launch_step_by_dim(step, aligned, merge_threads == 128 ? 128 : 256, smem, st);
+                rc = launch_step_by_dim(step, aligned, step_threads, smem, st);
                 if (rc < 0) return rc;
                 if (prof) VL_HIP(hipEventRecord(ev[3 * r + 1], st));
                 continue;
@@ -1478,7 +2045,8 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
             VL_HIP(hipMemcpyAsync(&sketch_rows, &ctrl->sketch_rows, sizeof(int), hipMemcpyDeviceToHost, st));
         VL_HIP(hipStreamSynchronize(st));
         if (prof) {
-            for (int r = 0; r < R; ++r) {
+            const int timed = launches ? launches : R;
+            for (int r = 0; r < timed; ++r) {
                 float ms = 0;
                 VL_HIP(hipEventElapsedTime(&ms, ev[3 * r], ev[3 * r + 1]));
                 mine.expand_ms += ms;
@@ -1487,8 +2055,8 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
                     mine.merge_ms += ms;
                 }
             }
-            mine.expand_launches += R;
-            mine.merge_launches += R;
+            mine.expand_launches += timed;
+            mine.merge_launches += timed;
         }
         if (!changed) break;  // ann.py:90-91
         if (t > t_limit) {
@@ -1611,6 +2179,8 @@ VL_EXPORT int vl_closest_vectors_noalloc(const vl_beam_params *p, const float *q
 // candidate distances asked for (fetched + served by the per-row cache),
 // out[8] = candidate rows looked at through the sketch, summed since the last
 // reset.
+VL_EXPORT int64_t vl_beam_launches(void) { return g_step_launches.load(std::memory_order_relaxed); }
+
 VL_EXPORT int vl_beam_profile(int enable, int reset, double *out) {
     std::lock_guard<std::mutex> hold(g_prof_mutex);
     if (out) {

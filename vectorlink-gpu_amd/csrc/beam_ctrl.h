@@ -33,7 +33,10 @@ struct BeamCtrl {
 //   0  normal
 // `writer` is true for exactly one thread of the launch, which records stop
 // and clears the ring slot of the next checking iteration.
-__device__ inline int beam_gate(BeamCtrl *c, int t, int R, int E, bool writer) {
+// look_at_fill = false (a launch that takes rows through several iterations, none of which can find a
+// visited list full): state 1 is not looked for - rows of such a launch that finish early raise the slot of
+// `first` that the launch after it reads, which for some lengths is the slot of iteration t - 1 modulo 3.
+__device__ inline int beam_gate(BeamCtrl *c, int t, int R, int E, bool writer, bool look_at_fill = true) {
     int stop = c->stop;
     const bool after_check = t > 1 && ((t - 1) % R) == 0;
     if (!stop && after_check && c->changed[((t - 1) / R) & 63] == 0) {
@@ -47,6 +50,6 @@ __device__ inline int beam_gate(BeamCtrl *c, int t, int R, int E, bool writer) {
     // the slot of the check after next: this iteration itself may be a checking one (R == 1)
     // and rows of one launch set their flag while others are still here
     if (writer && ((t - 1) % R) == 0) c->changed[((t - 1) / R + 2) & 63] = 0;
-    if (t >= 2 && c->first[(t - 1) % 3] >= E) return 1;
+    if (look_at_fill && t >= 2 && c->first[(t - 1) % 3] >= E) return 1;
     return 0;
 }

@@ -29,9 +29,11 @@ __device__ __forceinline__ uint32_t memo_hash(int32_t id, int shift) {
     const uint32_t group = (((uint32_t)id >> 4) * 2654435761u) >> shift;
     return (group & ~15u) | ((uint32_t)id & 15u);
 }
+__device__ __forceinline__ uint64_t memo_entry(int32_t id, float d) {
+    return ((uint64_t)__builtin_bit_cast(uint32_t, d) << 32) | (uint32_t)id;
+}
 __device__ __forceinline__ void memo_store(uint64_t *memo_row, int shift, int32_t id, float d) {
-    uint64_t e = ((uint64_t)__builtin_bit_cast(uint32_t, d) << 32) | (uint32_t)id;
-    __hip_atomic_store(memo_row + memo_hash(id, shift), e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(memo_row + memo_hash(id, shift), memo_entry(id, d), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ uint64_t memo_load(const uint64_t *memo_row, int shift, int32_t id) {
     return __hip_atomic_load(memo_row + memo_hash(id, shift), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -41,16 +43,34 @@ __device__ __forceinline__ uint64_t memo_load(const uint64_t *memo_row, int shif
 // bounds lo <= d <= hi as 16-bit fixed point, each moved one step outwards so that encoding and decoding
 // never narrow them.
 constexpr uint32_t kMemoBounds = 0x80000000u;
-__device__ __forceinline__ void memo_store_bounds(uint64_t *memo_row, int shift, int32_t id, float lo, float hi) {
+__device__ __forceinline__ uint64_t memo_bounds_entry(int32_t id, float lo, float hi) {
     int l = lo >= 0.0f ? (int)(lo * 65535.0f) - 1 : 0;   // a NaN bound becomes the widest one
     int h = hi <= 1.0f ? (int)(hi * 65535.0f) + 2 : 65535;
     l = l < 0 ? 0 : l;
     h = h > 65535 ? 65535 : h;
-    uint64_t e = ((uint64_t)(((uint32_t)l << 16) | (uint32_t)h) << 32) | ((uint32_t)id | kMemoBounds);
-    __hip_atomic_store(memo_row + memo_hash(id, shift), e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return ((uint64_t)(((uint32_t)l << 16) | (uint32_t)h) << 32) | ((uint32_t)id | kMemoBounds);
+}
+__device__ __forceinline__ void memo_store_bounds(uint64_t *memo_row, int shift, int32_t id, float lo, float hi) {
+    __hip_atomic_store(memo_row + memo_hash(id, shift), memo_bounds_entry(id, lo, hi), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ float memo_bound_lo(uint64_t e) { return (float)(uint32_t)(e >> 48) * (1.0f / 65535.0f); }
 __device__ __forceinline__ float memo_bound_hi(uint64_t e) { return (float)((uint32_t)(e >> 32) & 0xffffu) * (1.0f / 65535.0f); }
+
+// The same entries in a small direct-mapped table in LDS (a workgroup that takes a row through several
+// iterations keeps one): a repeat inside those iterations never leaves the compute unit.  An entry moves as one
+// 8-byte LDS access; shift = 32 - log2(slots); tab == nullptr: no table.
+struct LdsMemo {
+    uint64_t *tab;
+    int shift;
+};
+__device__ __forceinline__ uint32_t lds_memo_slot(int32_t id, int shift) { return ((uint32_t)id * 2654435761u) >> shift; }
+__device__ __forceinline__ uint64_t lds_memo_load(const LdsMemo &t, int32_t id) {
+    return __hip_atomic_load(t.tab + lds_memo_slot(id, t.shift), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ void lds_memo_store(const LdsMemo &t, int32_t id, uint64_t e) {
+    __hip_atomic_store(t.tab + lds_memo_slot(id, t.shift), e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
 
 // Folds the partial sums of a group of LPR lanes: lane l += lane l + h for h = LPR/2 ... 1, so the
 // group's first lane ends with the sum in the fixed order.  Steps of 32 and 16 lanes swap register
@@ -89,7 +109,7 @@ __device__ __forceinline__ void wave_distances(const float *__restrict__ q_row,
                                                const float *__restrict__ vectors, int dim,
                                                int nchunks, int32_t my_id, bool ok,
                                                float *__restrict__ out_d, uint64_t *memo_row,
-                                               int memo_shift, bool l2 = false) {
+                                               int memo_shift, bool l2 = false, LdsMemo lds = LdsMemo{nullptr, 0}) {
     constexpr int G = kWave / LPR;
     const int lane = threadIdx.x & (kWave - 1);
     const int grp = lane / LPR;
@@ -186,6 +206,7 @@ __device__ __forceinline__ void wave_distances(const float *__restrict__ q_row,
                 float d = finish_distance(acc, l2);
                 out_d[mysrc[u]] = d;
                 if (memo_row) memo_store(memo_row, memo_shift, ids[u], d);
+                if (lds.tab) lds_memo_store(lds, ids[u], memo_entry(ids[u], d));
             }
         }
     }

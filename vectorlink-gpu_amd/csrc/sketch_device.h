@@ -103,7 +103,8 @@ template <int SCPL, int SLPR, int SU>
 __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const uint8_t *__restrict__ table,
                                             const uint8_t *__restrict__ tails, int data_chunks, int32_t my_id, bool ok,
                                             float *__restrict__ out_lo, float *__restrict__ out_hi,
-                                            uint64_t *memo_row = nullptr, int memo_shift = 0) {
+                                            uint64_t *memo_row = nullptr, int memo_shift = 0,
+                                            LdsMemo lds = LdsMemo{nullptr, 0}) {
     constexpr int G = kWave / SLPR;
     const int lane = threadIdx.x & (kWave - 1);
     const int grp = lane / SLPR;
@@ -168,6 +169,7 @@ __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const u
                 out_lo[mysrc[u]] = lo;
                 out_hi[mysrc[u]] = hi;
                 if (memo_row) memo_store_bounds(memo_row, memo_shift, ids[u], lo, hi);
+                if (lds.tab) lds_memo_store(lds, ids[u], memo_bounds_entry(ids[u], lo, hi));
             }
         }
     }

@@ -61,6 +61,7 @@ _SIGNATURES = {
     "vl_sketch_bounds_workspace_bytes": (C.c_int64, [_i64, _i64]),
     "vl_sketch_bounds": (C.c_int, [_ptr, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr]),
     "vl_beam_profile": (C.c_int, [C.c_int, C.c_int, C.POINTER(C.c_double)]),
+    "vl_beam_launches": (C.c_int64, []),
     "vl_optimize_graph_workspace_bytes": (C.c_int64, [_i64, _i64, _i64]),
     "vl_optimize_graph": (C.c_int, [_ptr, _i64, _i64, _i64, _ptr, _ptr, _i64, _ptr]),
     "vl_knn_workspace_bytes": (C.c_int64, [_i64, _i64, _i64, _i64]),

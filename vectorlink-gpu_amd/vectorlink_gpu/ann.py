@@ -28,6 +28,7 @@ BEAM_SORT_MERGE = 2    # include/vlgpu.h: VL_BEAM_SORT_MERGE
 BEAM_PER_QUERY_STOP = 4  # include/vlgpu.h: VL_BEAM_PER_QUERY_STOP (a different loop: every row stops on its own)
 BEAM_NO_CACHE = 8  # include/vlgpu.h: VL_BEAM_NO_CACHE (no per-row cache of evaluated distances; same result)
 BEAM_USES_SKETCH = 16  # include/vlgpu.h: VL_BEAM_USES_SKETCH (set by closest_vectors when it is given a sketch)
+BEAM_WINDOWS = 32  # include/vlgpu.h: VL_BEAM_WINDOWS (several iterations per launch while rows are independent; same result)
 
 
 def _beam_params(batch: int, dim: int, n_vectors: int, width: int, queue: Queue, config: Dict,
