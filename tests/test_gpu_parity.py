@@ -400,6 +400,54 @@ def test_windows_with_rows_that_start_late_in_a_launch(ra):
     assert np.array_equal(bits(host(gq.distances)[:, :ql]), bits(oq.distances[:, :ql]))
 
 
+@pytest.mark.parametrize("dim,sketch", [(32, False), (64, False), (256, True)])
+def test_neighbour_lists_that_share_ids(dim, sketch):
+    """A ring graph (node i lists i+1 ... i+W): the four nodes a row visits in one iteration list mostly the
+    same ids.  Only one copy of an id is evaluated per iteration - the counters show it, with the distance
+    cache off so that nothing else answers a repeat - and the queues equal the oracle's, which evaluates
+    every copy as the reference does (kernels.py:238-255)."""
+    say(f"neighbour lists that share ids, dim={dim} sketch={sketch}")
+    import ctypes
+
+    from vectorlink_gpu import Queue
+    from vectorlink_gpu import _native as nv
+    from vectorlink_gpu.ann import BEAM_NO_CACHE, closest_vectors, excluding_self
+    from vectorlink_gpu.kernels import build_sketch
+
+    rng = np.random.default_rng(99 + dim)
+    n, beam, bqf, pv = 3000, 8, 2, 4
+    # rows that change slowly along the ring, so that a search walks along it and keeps visiting neighbours
+    steps = rng.standard_normal((n, dim)).astype(np.float32) * 0.05
+    v = np.cumsum(steps, axis=0) + rng.standard_normal(dim).astype(np.float32)
+    v = (v / np.linalg.norm(v, axis=1, keepdims=True)).astype(np.float32)
+    c = cfg(beam_size=beam, beam_queue_factor=bqf, parallel_visit_count=pv)
+    ql = beam * bqf
+    ring = ((np.arange(n, dtype=np.int64)[:, None] + np.arange(1, ql + 1)[None, :]) % n).astype(np.int32)
+    d = orc.calculate_distances(v, ring)
+    lo, hi = 100, 1300
+    oq = orc.Queue(hi - lo, ql, ql + ql * pv)
+    oq.insert(ring[lo:hi], d[lo:hi])
+    t_want = orc.closest_vectors(v[lo:hi], oq, v, ring, c, orc.excluding_self(lo, hi))
+    gv, gb = dev(v), dev(ring)
+    gq = Queue(hi - lo, ql, ql + ql * pv)
+    gq.insert(gb[lo:hi], dev(d)[lo:hi])
+    out = (ctypes.c_double * 9)()
+    nv.lib().vl_beam_profile(1, 1, out)
+    try:
+        t_got = closest_vectors(gv[lo:hi], gq, gv, gb, c, excluding_self(lo, hi), flags=BEAM_NO_CACHE,
+                                sketch=build_sketch(gv) if sketch else None)
+    finally:
+        nv.lib().vl_beam_profile(0, 1, out)
+    (fetched, wanted, sketched) = (out[4], out[7], out[8])
+    say(f"  iterations {t_got}, candidates {wanted:.0f}, through the sketch {sketched:.0f}, rows fetched {fetched:.0f}")
+    assert t_got == t_want
+    assert np.array_equal(host(gq.indices)[:, :ql], oq.indices[:, :ql])
+    assert np.array_equal(bits(host(gq.distances)[:, :ql]), bits(oq.distances[:, :ql]))
+    # four overlapping lists of 16 hold at most 19 + ... distinct ids of 64: well under half are looked at
+    looked_at = sketched + fetched if sketch else fetched
+    assert 0 < looked_at < 0.6 * wanted
+
+
 def test_generate_ann_and_search_against_oracle():
     say("generate_ann + search, n=1500")
     from vectorlink_gpu import ANN

@@ -895,6 +895,15 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
         probe_hits_s = 0;
         probe_asked_s = 0;
     }
+    // The neighbour lists of the nodes visited in one iteration share ids; only one copy of an id is evaluated.
+    // Every candidate claims its id in a hash set in LDS (the merge phase's array for filtered keys, free until
+    // then: 2 * Pc slots for at most m <= Pc ids, each the slot number of the claiming candidate); a candidate that
+    // finds its id claimed becomes the empty pair before anything is asked of memory for it.  The reference
+    // evaluates every copy (kernels.py:238-255) and drops all but one when the queues are sorted
+    // (kernels.py:314-349): copies carry the same distance, so what the queues receive is the same.
+    int32_t *const dset = reinterpret_cast<int32_t *>(uk + a.Pc);
+    const uint32_t dmask = 2u * (uint32_t)a.Pc - 1u;
+    for (int i = tid; i < 2 * a.Pc; i += THREADS) dset[i] = -1;
     __syncthreads();
 
     // ---- expand: ann.py:69-73 (pop the visit heads, gather their neighbour lists, distances) ----
@@ -945,21 +954,40 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
     int n_wanted = 0, n_fetched = 0, n_sketched = 0;  // counts of this wavefront
     float *le = reinterpret_cast<float *>(raw);                     // upper bounds (raw is filled in the merge phase)
     uint8_t *xf = reinterpret_cast<uint8_t *>(exl + a.excl_cols);   // the merge phase's per-candidate flags; 16 = exact
+    // first pass over this wavefront's candidates: ids to LDS, later copies of an id out
+    for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
+        if (c0 != wave * kWave) id = resolve(c0);
+        const int slot = c0 + lane;
+        const bool has = slot < a.m;
+        bool ok = has && id != VL_MAXINT && id >= 0 && (int64_t)id < s.n_vectors;
+        if (s.count_evals || resample) n_wanted += __popcll(__ballot(ok));
+        if (has) li[slot] = ok ? id : VL_MAXINT;  // (before the claim: a candidate that meets this one in the set reads it)
+        if (ok) {
+            uint32_t h = ((uint32_t)id * 2654435761u) >> 7;
+            for (;;) {
+                h &= dmask;
+                const int owner = atomicCAS(&dset[h], -1, slot);
+                if (owner == -1) break;     // first of its id
+                if (li[owner] == id) {      // a copy: only the first is evaluated
+                    ok = false;
+                    break;
+                }
+                ++h;
+            }
+            if (!ok) li[slot] = VL_MAXINT;
+        }
+        if (has && !ok) ld[slot] = VL_MAXFLOAT;
+    }
     if constexpr (SCPL > 0) {
         if (sketching) {
             SketchQuery<SCPL> sq;
             sketch_query_load<SCPL, SLPR>(sq, s.rounded_queries + row * s.rounded_query_bytes, s.sketch_chunks);
             for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
-                if (c0 != wave * kWave) id = resolve(c0);
                 const int slot = c0 + lane;
                 const bool has = slot < a.m;
-                bool ok = has && id != VL_MAXINT && id >= 0 && (int64_t)id < s.n_vectors;
-                if (has) {
-                    li[slot] = ok ? id : VL_MAXINT;
-                    if (!ok) ld[slot] = VL_MAXFLOAT;
-                    xf[slot] = 0;
-                }
-                if (s.count_evals || resample) n_wanted += __popcll(__ballot(ok));
+                id = has ? li[slot] : VL_MAXINT;
+                bool ok = id != VL_MAXINT;
+                if (has) xf[slot] = 0;
                 // The cache serves two kinds of repeats: a candidate evaluated exactly before comes back with its
                 // distance, one that was only bounded comes back with its bounds (dist_device.h) - either way
                 // nothing is fetched for it now.
@@ -986,15 +1014,10 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
         }
     }
     for (int c0 = wave * kWave; c0 < a.m && !sketching; c0 += THREADS) {
-        if (c0 != wave * kWave) id = resolve(c0);
         const int slot = c0 + lane;
         const bool has = slot < a.m;
-        bool ok = has && id != VL_MAXINT && id >= 0 && (int64_t)id < s.n_vectors;
-        if (has) {
-            li[slot] = ok ? id : VL_MAXINT;
-            if (!ok) ld[slot] = VL_MAXFLOAT;
-        }
-        if (s.count_evals || resample) n_wanted += __popcll(__ballot(ok));
+        id = has ? li[slot] : VL_MAXINT;
+        bool ok = id != VL_MAXINT;
         if (probing && ok) {
             uint64_t e = memo_load(memo_row, s.memo_shift, id);
             if ((int32_t)(uint32_t)e == id) {
