@@ -78,6 +78,59 @@ def test_build_1m_x_128_properties(mix128):
     assert torch.equal(r3.indices[:, :r3.length], r1.indices[:, :r1.length])
 
 
+def test_build_1m_x_768_properties():
+    """The headline workload built whole (1M x 768, degree 64, queue 128, three loops with the reference's
+    prune, through cache + sketch): what can be checked without the oracle at that size."""
+    say("full build 1M x 768")
+    from vectorlink_gpu import ANN, synthetic
+    from vectorlink_gpu.kernels import gather_distances, knn_exact
+
+    base, q, w = synthetic.make("mix-1m-768")
+    v = base.to(DEV)
+    ann = ANN(v, **synthetic.ann_kwargs(w))
+    n, deg = ann.beams.shape
+    assert (n, deg) == (1_000_000, 64) and ann.distances.shape == (n, deg)
+    ids, d = ann.beams, ann.distances
+    real = ids != M
+    assert bool(real[:, 0].all())
+    assert bool(((ids >= 0) & (ids < n))[real].all())
+    rows = torch.arange(n, device=DEV, dtype=torch.int32).unsqueeze(1).expand(n, deg)
+    assert not bool((ids == rows)[real].any())                       # no self edges
+    assert bool((d[:, 1:] >= d[:, :-1]).all())                        # rows ordered by distance
+    srt = ids.sort(dim=1).values
+    assert not bool(((srt[:, 1:] == srt[:, :-1]) & (srt[:, 1:] != M)).any())  # distinct ids per row
+    assert bool((d[~real] == torch.tensor(3.4028e37, device=DEV)).all())
+    del srt, rows
+    # the distances are the distances of the ids: recomputed bit for bit, and against float64 on a sample
+    again = gather_distances(v, v, ids)
+    assert torch.equal(again, d)
+    del again
+    sample = torch.randint(0, n, (256,), generator=torch.Generator(device="cpu").manual_seed(0), device="cpu")
+    vs = base[sample].double()
+    nb = base[ids[sample.to(DEV)].cpu().long().clamp(max=n - 1)].double()     # [256, deg, dim]
+    ref = ((1 - (vs.unsqueeze(1) * nb).sum(2)) / 2).clamp(0, 1)
+    ok = real[sample.to(DEV)].cpu()
+    assert torch.allclose(d[sample.to(DEV)].cpu().double()[ok], ref[ok], rtol=1e-5, atol=1e-6)
+    # graph quality: most of a row's exact 10 nearest neighbours are among its 64
+    t11, _ = knn_exact(v[:1024].contiguous(), v, 11)
+    hits = (ids[:1024, :, None] == t11[:, None, 1:11]).any(dim=1).sum().item()
+    say(f"  exact 10-NN among the 64 neighbours: {hits / (1024 * 10):.3f}")
+    assert hits / (1024 * 10) > 0.85
+    # search: deterministic, ordered, real distances of real ids, recall@10 at the quoted level
+    qd = q[:2000].to(DEV)
+    r1 = ann.search(qd, seeding="dense")
+    r2 = ann.search(qd, seeding="dense")
+    assert torch.equal(r1.indices[:, :r1.length], r2.indices[:, :r2.length])
+    assert bool((r1.distances[:, 1:r1.length] >= r1.distances[:, :r1.length - 1]).all())
+    truth, td = knn_exact(qd, v, 10)
+    found = r1.indices[:, :10]
+    recall = (found.unsqueeze(2) == truth.unsqueeze(1)).any(dim=2).sum().item() / truth.numel()
+    say(f"  recall@10 with dense seeds: {recall:.4f}")
+    assert recall >= 0.95
+    fd = gather_distances(qd, v, found.contiguous())
+    assert torch.equal(fd, r1.distances[:, :10])
+
+
 def test_1m_x_768_distances_knn_and_one_batch_on_the_oracle():
     say("1M x 768: distances, exact kNN, one small batch against the oracle")
     from vectorlink_gpu import synthetic
@@ -376,3 +429,19 @@ def test_sketch_and_plain_paths_agree_at_scale(workload, n):
             assert sketched > 0
         if state == 0:
             assert results[1][3] < 0.5 * fetched0 and results[2][3] < 0.5 * fetched0
+        # 24 rows of the same state through cache + sketch, replayed on the CPU oracle: exact ids and distances
+        # (state 1 is what 45 % of a build's launches run on: a pruned table with empty slots, distances carried)
+        few = 24
+        q = Queue(few, ql, ql + ql * c["parallel_visit_count"], device=DEV)
+        q.insert(tb[n - few:], td[n - few:])
+        t_gpu = closest_vectors(v[n - few:], q, v, tb, c, excluding_self(n - few, n, device=DEV), sketch=sk)
+        vn, tbn, tdn = base.numpy(), tb.cpu().numpy(), td.cpu().numpy()
+        oq = orc.Queue(few, ql, ql + ql * c["parallel_visit_count"])
+        oq.insert(tbn[n - few:], tdn[n - few:])
+        t_cpu = orc.closest_vectors(vn[n - few:], oq, vn, tbn, c, orc.excluding_self(n - few, n))
+        say(f"  state {state}: {few} rows on the oracle, {t_cpu} iterations")
+        assert t_gpu == t_cpu
+        assert np.array_equal(q.indices[:, :ql].cpu().numpy(), oq.indices[:, :ql])
+        assert np.array_equal(q.distances[:, :ql].cpu().numpy().view(np.uint32), oq.distances[:, :ql].view(np.uint32))
+        if state == 1:
+            assert (tbn == M).any()
