@@ -312,10 +312,14 @@ int64_t vl_closest_vectors_with_sketch(const vl_beam_params *p,
  *    remaining launches do nothing, so with iterations >= the count
  *    vl_closest_vectors would return the queues end up bit-identical to its;
  *  - status_out (device, 2 x int32) receives [0] = 1 if the loop ended within
- *    `iterations` (else 0: the queues hold an unfinished search) and [1] = the
- *    number of iterations that ran.
+ *    `iterations` (else 0: the queues hold an unfinished search; -1: a row found
+ *    more ids in its visited list than the iterations run can have put there,
+ *    i.e. the array was written by another call meanwhile - the rows stop and
+ *    the queues are not to be used) and [1] = the number of iterations that ran.
  * All calls on one GPU share that GPU's array: calls that overlap on one GPU
- * (two streams, two threads) race; serialise them. */
+ * (two streams, two threads) race; serialise them.  (vl_closest_vectors reports
+ * the same condition, a workspace shared by two calls in flight, as
+ * VL_ERR_STATE.) */
 #define VL_NOALLOC_SCRATCH_BYTES (32 << 20)
 int vl_closest_vectors_noalloc(const vl_beam_params *p,
                                const float *queries, const float *vectors,

@@ -594,6 +594,26 @@ def test_optimize_graph(n, w, d):
     assert np.array_equal(got, want)
 
 
+def test_optimize_graph_with_hubs():
+    """Rows that thousands of others point at from their first slots: the reverse pass keeps only the first few
+    sources of a row in (slot, source) order and must find them among more edges than it sorts at a time,
+    whatever order the edges were scattered in."""
+    say("optimize_graph with hubs")
+    from vectorlink_gpu.kernels import optimize_graph
+
+    rng = np.random.default_rng(8)
+    n, w, d = 6000, 12, 8
+    beams = np.stack([rng.choice(n, size=w, replace=False) for _ in range(n)]).astype(np.int32)
+    beams[:, 0] = 7                      # every row points at row 7 from slot 0 ...
+    beams[::2, 1] = 11                   # ... half of them at row 11 from slot 1 ...
+    beams[rng.random(n) < 0.3, 2] = 7    # ... and some at row 7 again from slot 2 (an id twice in a row)
+    beams[7, 0], beams[11, 1] = 8, 12
+    want = orc.optimize_graph(beams, d)
+    for _ in range(3):                   # the scatter's order differs from run to run; the result must not
+        got = host(optimize_graph(dev(beams), d))
+        assert np.array_equal(got, want)
+
+
 def test_rank_pruned_build():
     say("build with prune='rank'")
     from vectorlink_gpu import ANN

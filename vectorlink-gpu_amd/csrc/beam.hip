@@ -125,6 +125,7 @@ __global__ __launch_bounds__(kQueueThreads) void beam_init_kernel(BeamCtrl *ctrl
         ctrl->ended_after = 0;
         ctrl->first[0] = ctrl->first[1] = ctrl->first[2] = 0;
         ctrl->sketch_rows = sketch_rows;
+        ctrl->error = 0;
     }
     if (t < 64) ctrl->changed[t] = 0;
     if (t < kBeamStripes) {
@@ -538,6 +539,9 @@ __device__ __forceinline__ MergeResult merge_row(const MergeArgs &a, unsigned ch
         }
     }
     if (stop) return MergeResult{cnt, false};
+    if constexpr (!FUSED) {
+        if (!beam_row_state_ok(c, cnt, min(a.E, a.Vt * (t - 1)), threadIdx.x == 0)) return MergeResult{0, false};
+    }
     if (!FUSED && t >= 2 && first_prev >= a.E) {
         // the visit queue is no longer fed: every candidate of this iteration is empty
         if (threadIdx.x == 0) raise_running_max(first_next, cnt, min(a.E, a.Vt * t));
@@ -863,6 +867,7 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
 
     const int gate = beam_gate(c, t, a.readahead, a.E, blockIdx.x == 0 && tid == 0);
     if (gate == 2) return;
+    if (!beam_row_state_ok(c, pre.cnt, seen_bound, tid == 0)) return;
     if (gate == 1 || (a.row_quiet && quiet >= a.readahead)) {
         // the visit queue is no longer fed (every candidate of this iteration is empty), or this row has
         // stopped on its own: nothing changes, only the running maximum is kept current
@@ -1232,6 +1237,7 @@ __device__ __forceinline__ void beam_window_body(const StepArgs &s) {
     // of this very launch that finish early write the one the next launch reads)
     const int gate = beam_gate(c, t0, a.readahead, a.E, blockIdx.x == 0 && tid == 0, false);
     if (gate == 2) return;
+    if (!beam_row_state_ok(c, cnt, seen_bound, tid == 0)) return;
     int *first_after = &c->first[(t0 + W) % 3];  // what the launch of iteration t0 + W reads
     const int bound_after = min(a.E, a.Vt * (t0 + W - 1));
     if (a.row_quiet && quiet0 >= a.readahead) {
@@ -1811,7 +1817,7 @@ __global__ void beam_status_kernel(const BeamCtrl *c, int iterations, int R, int
         ended = 1;  // the last launch was a checking iteration that found every row quiet
         t = iterations;
     }
-    status[0] = ended;
+    status[0] = c->error ? -1 : ended;  // -1: a row's state was impossible (the scratch memory was shared with another call)
     status[1] = ended ? t : iterations;
 }
 
@@ -2063,10 +2069,16 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
             if (prof) VL_HIP(hipEventRecord(ev[3 * r + 2], st));
         }
         int changed = 0;
+        int state[2] = {0, 0};  // sketch_rows, error (neighbours in the control block)
         VL_HIP(hipMemcpyAsync(&changed, &ctrl->changed[(t / R) & 63], sizeof(int), hipMemcpyDeviceToHost, st));
-        if (sketch_table)
-            VL_HIP(hipMemcpyAsync(&sketch_rows, &ctrl->sketch_rows, sizeof(int), hipMemcpyDeviceToHost, st));
+        VL_HIP(hipMemcpyAsync(state, &ctrl->sketch_rows, sizeof(state), hipMemcpyDeviceToHost, st));
         VL_HIP(hipStreamSynchronize(st));
+        if (sketch_table) sketch_rows = state[0];
+        if (state[1]) {
+            vl_set_error("a row's visited list holds more ids than %lld iterations can have put there: the workspace "
+                         "was overwritten while the loop ran - is it shared with a concurrent call?", (long long)t);
+            return VL_ERR_STATE;
+        }
         if (prof) {
             const int timed = launches ? launches : R;
             for (int r = 0; r < timed; ++r) {

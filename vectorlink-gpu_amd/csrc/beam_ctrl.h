@@ -9,6 +9,7 @@
 //                 kept sorted
 //   changed[64] - ring of "some row changed" flags, one per checking iteration
 //   sketch_rows - how many rows currently use the 8-bit sketch (they opt in once and may opt out once)
+//   error       - a row found its own state impossible (see beam_row_state_ok)
 #pragma once
 #include "vl_common.h"
 
@@ -20,11 +21,25 @@ struct BeamCtrl {
     int first[3];
     int changed[64];
     int sketch_rows;    // rows that currently look at their candidates through the 8-bit sketch first
+    int error;          // set by a row whose visited-list fill is beyond what the iteration count allows: the
+                        // workspace was overwritten while the loop ran (VL_ERR_STATE on the host)
     // profiling only, striped by workgroup so that the atomic adds do not queue up on one address:
     unsigned long long evals[kBeamStripes];   // candidate rows actually fetched
     unsigned long long wanted[kBeamStripes];  // candidate distances asked for (fetched or served by the cache)
     unsigned long long sketched[kBeamStripes];  // candidate rows looked at through the 8-bit sketch only
 };
+
+// A row's visited list holds at most Vt ids per earlier iteration and never more than its E slots.  A
+// count beyond that was not written by this loop (its workspace is shared with another call): the row
+// must not run - its copy loops would run to that count - and the loop ends with an error.
+__device__ inline bool beam_row_state_ok(BeamCtrl *c, int cnt, int bound, bool writer) {
+    if (cnt >= 0 && cnt <= bound) return true;
+    if (writer) {
+        c->error = 1;
+        c->stop = 1;
+    }
+    return false;
+}
 
 // State of iteration t as seen by a kernel launched for it:
 //   2  the loop has ended, do nothing

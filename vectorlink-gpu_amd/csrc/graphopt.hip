@@ -10,20 +10,24 @@
 //                        y in row x, count a detour for that slot; re-order by
 //                        (detours, slot), keep `degree`.  W rows of W ids are
 //                        read per row (W^2 * 4 bytes, rows gathered).
-//  reverse edges         (y, slot) keys + x values for the first rev_from slots
-//                        of every pruned row, one stable radix sort (rocPRIM):
-//                        afterwards the sources of each y are contiguous and
-//                        ordered by (slot, x).
-//  reverse_merge_kernel  one workgroup per row: keep | reverse | rest, without
-//                        duplicates, cut to `degree`.
+//  reverse edges         the edges x -> y of the first rev_from slots of every
+//                        pruned row, grouped by target: a histogram of the
+//                        targets, an exclusive scan of it (three small
+//                        kernels), and a scatter of (slot, x) keys into the
+//                        targets' segments, in whatever order the atomics hand
+//                        out the places of a segment.
+//  reverse_merge_kernel  one workgroup per row y: only the first `cap` sources of
+//                        y in (slot, x) order are needed, and they are selected
+//                        from the segment here (chunks of it sorted in LDS
+//                        together with the best so far), so the result does not
+//                        depend on the segment's order; then keep | reverse |
+//                        rest, without duplicates, cut to `degree`.
 #include "rowsort.h"
 
 #include <cstring>
-#include <rocprim/device/device_radix_sort.hpp>
 
 namespace {
 
-constexpr int kSlotBits = 12;  // slots per row < 4096
 
 __global__ __launch_bounds__(kQueueThreads) void rank_prune_kernel(const int32_t *__restrict__ beams, int64_t n, int W,
                                                                   int P, int degree, int32_t *__restrict__ out,
@@ -72,50 +76,153 @@ __global__ __launch_bounds__(kQueueThreads) void rank_prune_kernel(const int32_t
     }
 }
 
-__global__ void rev_keys_kernel(const int32_t *__restrict__ pruned, int64_t n, int degree, int rev_from,
-                                uint64_t *__restrict__ keys, int32_t *__restrict__ vals) {
+// An edge of the reverse pass: slot k < rev_from of pruned row x, pointing at a real row y.
+__device__ inline bool rev_edge(const int32_t *__restrict__ pruned, int64_t n, int degree, int rev_from, int64_t e,
+                                int64_t *x, int *k, int32_t *y) {
+    *x = e / rev_from;
+    *k = (int)(e - *x * rev_from);
+    *y = pruned[*x * degree + *k];
+    return *y != VL_MAXINT && *y >= 0 && *y < n;
+}
+
+__global__ void rev_zero_kernel(int32_t *__restrict__ a, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) a[i] = 0;
+}
+
+// count[y] = edges that point at y
+__global__ void rev_count_kernel(const int32_t *__restrict__ pruned, int64_t n, int degree, int rev_from,
+                                 int32_t *__restrict__ count) {
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n * rev_from;
          e += (int64_t)gridDim.x * blockDim.x) {
-        int64_t x = e / rev_from;
-        int k = (int)(e - x * rev_from);
-        int32_t y = pruned[x * degree + k];
-        bool real = y != VL_MAXINT && y >= 0 && y < n;
-        keys[e] = real ? (((uint64_t)(uint32_t)y << kSlotBits) | (uint32_t)k) : ((1ull << (30 + kSlotBits)) | 0ull);
-        vals[e] = (int32_t)x;
+        int64_t x;
+        int k;
+        int32_t y;
+        if (rev_edge(pruned, n, degree, rev_from, e, &x, &k, &y)) atomicAdd(&count[y], 1);
     }
 }
 
-// start[y] = first sorted edge whose target is >= y, for y in [0, n]
-__global__ void rev_start_kernel(const uint64_t *__restrict__ keys, int64_t n_edges, int64_t n, int64_t *__restrict__ start) {
-    for (int64_t y = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; y <= n; y += (int64_t)gridDim.x * blockDim.x) {
-        uint64_t want = (uint64_t)y << kSlotBits;
-        int64_t lo = 0, hi = n_edges;
-        while (lo < hi) {
-            int64_t mid = (lo + hi) >> 1;
-            if (keys[mid] < want) lo = mid + 1;
-            else hi = mid;
-        }
-        start[y] = lo;
+// Exclusive scan of m counts in three steps: every workgroup scans kScanItems of them and reports its total,
+// one workgroup scans the totals, every workgroup adds the total of those before it.
+constexpr int kScanThreads = 256, kScanPerThread = 8, kScanItems = kScanThreads * kScanPerThread;
+
+__device__ inline int block_exclusive_scan(int mine, int *lds, int *total) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    int incl = mine;
+    for (int d = 1; d < kWave; d <<= 1) {
+        int up = __shfl_up(incl, d);
+        if (lane >= d) incl += up;
+    }
+    if (lane == kWave - 1) lds[wave] = incl;
+    __syncthreads();
+    int before = 0, all = 0;
+    for (int w = 0; w < (int)(blockDim.x / kWave); ++w) {
+        if (w < wave) before += lds[w];
+        all += lds[w];
+    }
+    __syncthreads();
+    *total = all;
+    return before + incl - mine;
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan_blocks_kernel(const int32_t *__restrict__ in, int64_t m,
+                                                                  int32_t *__restrict__ out,
+                                                                  int32_t *__restrict__ block_total) {
+    __shared__ int lds[kScanThreads / kWave];
+    const int64_t base = (int64_t)blockIdx.x * kScanItems + (int64_t)threadIdx.x * kScanPerThread;
+    int v[kScanPerThread], sum = 0;
+#pragma unroll
+    for (int j = 0; j < kScanPerThread; ++j) {
+        v[j] = base + j < m ? in[base + j] : 0;
+        sum += v[j];
+    }
+    int total;
+    int run = block_exclusive_scan(sum, lds, &total);
+#pragma unroll
+    for (int j = 0; j < kScanPerThread; ++j) {
+        if (base + j < m) out[base + j] = run;
+        run += v[j];
+    }
+    if (threadIdx.x == 0) block_total[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(1024) void scan_totals_kernel(int32_t *__restrict__ block_total, int64_t blocks) {
+    __shared__ int lds[1024 / kWave];
+    int carry = 0;
+    for (int64_t base = 0; base < blocks; base += 1024) {
+        const int64_t i = base + threadIdx.x;
+        const int v = i < blocks ? block_total[i] : 0;
+        int total;
+        const int ex = block_exclusive_scan(v, lds, &total);
+        if (i < blocks) block_total[i] = carry + ex;
+        carry += total;
     }
 }
+
+__global__ __launch_bounds__(kScanThreads) void scan_add_kernel(int32_t *__restrict__ out, int64_t m,
+                                                               const int32_t *__restrict__ block_total) {
+    const int add = block_total[blockIdx.x];
+    const int64_t base = (int64_t)blockIdx.x * kScanItems + threadIdx.x;
+    for (int j = 0; j < kScanPerThread; ++j) {
+        const int64_t i = base + (int64_t)j * kScanThreads;
+        if (i < m) out[i] += add;
+    }
+}
+
+// keys[start[y] ...] receive the (slot << 32 | x) of the edges that point at y; count[y] runs down to 0 as the
+// places of y's segment are handed out (from its end: the order inside a segment is whatever the atomics make it)
+__global__ void rev_scatter_kernel(const int32_t *__restrict__ pruned, int64_t n, int degree, int rev_from,
+                                   const int32_t *__restrict__ start, int32_t *__restrict__ count,
+                                   uint64_t *__restrict__ keys) {
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n * rev_from;
+         e += (int64_t)gridDim.x * blockDim.x) {
+        int64_t x;
+        int k;
+        int32_t y;
+        if (rev_edge(pruned, n, degree, rev_from, e, &x, &k, &y)) {
+            const int place = atomicSub(&count[y], 1) - 1;
+            keys[(int64_t)start[y] + place] = ((uint64_t)(uint32_t)k << 32) | (uint32_t)x;
+        }
+    }
+}
+
+constexpr int kRevChunk = 1024;  // keys of a segment sorted at a time, together with the best so far
 
 __global__ __launch_bounds__(kQueueThreads) void reverse_merge_kernel(const int32_t *__restrict__ pruned, int64_t n,
-                                                                     int degree, int keep, int cap,
-                                                                     const int32_t *__restrict__ rev_src,
-                                                                     const int64_t *__restrict__ start,
+                                                                     int degree, int keep, int cap, int best_slots,
+                                                                     const uint64_t *__restrict__ rev_keys,
+                                                                     const int32_t *__restrict__ start,
                                                                      int32_t *__restrict__ out, int64_t row0) {
     extern __shared__ __align__(16) unsigned char smem[];
-    int32_t *cand = reinterpret_cast<int32_t *>(smem);  // keep | reverse | rest
+    uint64_t *best = reinterpret_cast<uint64_t *>(smem);            // [0, cap): the smallest (slot, x) so far
+    int32_t *cand = reinterpret_cast<int32_t *>(best + best_slots);  // keep | reverse | rest
     uint8_t *ok = reinterpret_cast<uint8_t *>(cand + 2 * degree);
     __shared__ int wave_cnt[kQueueWaves];
     const int64_t x = row0 + blockIdx.x;
     const int64_t s = start[x];
-    const int n_rev = (int)min((int64_t)cap, start[x + 1] - s);
+    const int64_t seg = (int64_t)start[x + 1] - s;
+    const int n_rev = (int)min((int64_t)cap, seg);
+    // the first n_rev sources of x in (slot, source) order: chunk after chunk of the segment is sorted together
+    // with the best of the chunks before it; what ends up in [0, n_rev) is the same whatever order the segment is in
+    for (int64_t done = 0; done < seg; done += kRevChunk) {
+        const int len = (int)min((int64_t)kRevChunk, seg - done);
+        const int held = done == 0 ? 0 : cap;
+        int P = 2;
+        while (P < held + len) P <<= 1;
+        for (int i = threadIdx.x; i < P; i += blockDim.x) {
+            if (i >= held) best[i] = i - held < len ? rev_keys[s + done + (i - held)] : kPadKey;
+        }
+        block_bitonic_sort(best, P);
+        if (seg > kRevChunk) {  // more chunks may follow: everything beyond the best `cap` is forgotten
+            for (int i = cap + threadIdx.x; i < P; i += blockDim.x) best[i] = kPadKey;
+            for (int i = P + threadIdx.x; i < cap; i += blockDim.x) best[i] = kPadKey;
+            __syncthreads();
+        }
+    }
     const int total = keep + n_rev + (degree - keep);
     for (int p = threadIdx.x; p < total; p += blockDim.x) {
         int32_t v;
         if (p < keep) v = pruned[x * degree + p];
-        else if (p < keep + n_rev) v = rev_src[s + (p - keep)];
+        else if (p < keep + n_rev) v = (int32_t)(uint32_t)best[p - keep];
         else v = pruned[x * degree + keep + (p - keep - n_rev)];
         cand[p] = v;
     }
@@ -154,9 +261,8 @@ __global__ __launch_bounds__(kQueueThreads) void reverse_merge_kernel(const int3
 }
 
 struct OptPlan {
-    int64_t n_edges;
-    int64_t off_pruned, off_keys_a, off_keys_b, off_vals_a, off_vals_b, off_start, off_temp, total;
-    size_t temp_bytes;
+    int64_t n_edges, scan_blocks;
+    int64_t off_pruned, off_keys, off_count, off_start, off_totals, total;
     int rev_from, keep;
 };
 
@@ -169,26 +275,14 @@ int opt_plan(int64_t n, int64_t width, int64_t degree, OptPlan *p) {
     p->keep = (int)(degree / 2);
     p->rev_from = (int)(degree / 2);
     p->n_edges = n * p->rev_from;
-    VL_REQUIRE(p->n_edges < (1ll << 31), "too many reverse edges for one sort");
-    size_t temp = 0;
-    if (p->n_edges > 0) {
-        hipError_t e = rocprim::radix_sort_pairs(nullptr, temp, (uint64_t *)nullptr, (uint64_t *)nullptr,
-                                                 (int32_t *)nullptr, (int32_t *)nullptr, (size_t)p->n_edges, 0,
-                                                 31 + kSlotBits, (hipStream_t)0);
-        if (e != hipSuccess) {
-            vl_set_error("rocprim::radix_sort_pairs (size query) failed: %s", hipGetErrorString(e));
-            return VL_ERR_HIP;
-        }
-    }
-    p->temp_bytes = temp;
+    VL_REQUIRE(p->n_edges < (1ll << 31), "too many reverse edges for 32-bit segment offsets");
+    p->scan_blocks = (n + 1 + kScanItems - 1) / kScanItems;
     int64_t o = 0;
     p->off_pruned = o; o = align256(o + n * degree * 4);
-    p->off_keys_a = o; o = align256(o + p->n_edges * 8);
-    p->off_keys_b = o; o = align256(o + p->n_edges * 8);
-    p->off_vals_a = o; o = align256(o + p->n_edges * 4);
-    p->off_vals_b = o; o = align256(o + p->n_edges * 4);
-    p->off_start = o; o = align256(o + (n + 1) * 8);
-    p->off_temp = o; o = align256(o + (int64_t)temp);
+    p->off_keys = o; o = align256(o + p->n_edges * 8);
+    p->off_count = o; o = align256(o + (n + 1) * 4);
+    p->off_start = o; o = align256(o + (n + 1) * 4);
+    p->off_totals = o; o = align256(o + p->scan_blocks * 4);
     p->total = o;
     return VL_OK;
 }
@@ -216,9 +310,9 @@ VL_EXPORT int vl_optimize_graph(const int32_t *beams, int64_t n, int64_t width, 
     hipStream_t st = (hipStream_t)stream;
     char *ws = (char *)workspace;
     int32_t *pruned = (int32_t *)(ws + p.off_pruned);
-    uint64_t *keys_a = (uint64_t *)(ws + p.off_keys_a), *keys_b = (uint64_t *)(ws + p.off_keys_b);
-    int32_t *vals_a = (int32_t *)(ws + p.off_vals_a), *vals_b = (int32_t *)(ws + p.off_vals_b);
-    int64_t *start = (int64_t *)(ws + p.off_start);
+    uint64_t *keys = (uint64_t *)(ws + p.off_keys);
+    int32_t *count = (int32_t *)(ws + p.off_count), *start = (int32_t *)(ws + p.off_start);
+    int32_t *totals = (int32_t *)(ws + p.off_totals);
 
     int P = vl_next_pow2(width);
     if (P < 2) P = 2;
@@ -230,22 +324,33 @@ VL_EXPORT int vl_optimize_graph(const int32_t *beams, int64_t n, int64_t width, 
     }
     VL_LAUNCH_CHECK("rank_prune_kernel");
 
+    // the reverse edges grouped by target: histogram, exclusive scan, scatter
+    hipLaunchKernelGGL(rev_zero_kernel, dim3(vl_grid_for(n + 1, 256)), dim3(256), 0, st, count, n + 1);
+    VL_LAUNCH_CHECK("rev_zero_kernel");
     if (p.n_edges > 0) {
-        hipLaunchKernelGGL(rev_keys_kernel, dim3(vl_grid_for(p.n_edges, 256)), dim3(256), 0, st, pruned, n,
-                           (int)degree, p.rev_from, keys_a, vals_a);
-        VL_LAUNCH_CHECK("rev_keys_kernel");
-        size_t temp = p.temp_bytes;
-        VL_HIP(rocprim::radix_sort_pairs(ws + p.off_temp, temp, keys_a, keys_b, vals_a, vals_b, (size_t)p.n_edges, 0,
-                                         31 + kSlotBits, st));
+        hipLaunchKernelGGL(rev_count_kernel, dim3(vl_grid_for(p.n_edges, 256)), dim3(256), 0, st, pruned, n, (int)degree,
+                           p.rev_from, count);
+        VL_LAUNCH_CHECK("rev_count_kernel");
     }
-    hipLaunchKernelGGL(rev_start_kernel, dim3(vl_grid_for(n + 1, 256)), dim3(256), 0, st, keys_b, p.n_edges, n,
-                       start);
-    VL_LAUNCH_CHECK("rev_start_kernel");
-    size_t smem2 = (size_t)degree * 8 + (size_t)degree * 2 + 16;
+    hipLaunchKernelGGL(scan_blocks_kernel, dim3((unsigned)p.scan_blocks), dim3(kScanThreads), 0, st, count, n + 1, start,
+                       totals);
+    hipLaunchKernelGGL(scan_totals_kernel, dim3(1), dim3(1024), 0, st, totals, p.scan_blocks);
+    hipLaunchKernelGGL(scan_add_kernel, dim3((unsigned)p.scan_blocks), dim3(kScanThreads), 0, st, start, n + 1, totals);
+    VL_LAUNCH_CHECK("exclusive scan of the edge counts");
+    if (p.n_edges > 0) {
+        hipLaunchKernelGGL(rev_scatter_kernel, dim3(vl_grid_for(p.n_edges, 256)), dim3(256), 0, st, pruned, n, (int)degree,
+                           p.rev_from, start, count, keys);
+        VL_LAUNCH_CHECK("rev_scatter_kernel");
+    }
+    const int cap = (int)(degree - p.keep);
+    // the sort of a chunk together with the best so far pads to a power of two (at most 4096 slots: cap <= 1024)
+    const int best_slots = vl_next_pow2(cap + kRevChunk);
+    const size_t smem2 = (size_t)best_slots * 8 + (size_t)degree * 8 + (size_t)degree * 2 + 16;
+    VL_HIP(vl_allow_lds(reverse_merge_kernel, smem2));
     for (int64_t row0 = 0; row0 < n; row0 += kMaxBlocks) {
         int64_t rows = n - row0 < kMaxBlocks ? n - row0 : kMaxBlocks;
         hipLaunchKernelGGL(reverse_merge_kernel, dim3((unsigned)rows), dim3(kQueueThreads), smem2, st, pruned, n,
-                           (int)degree, p.keep, (int)(degree - p.keep), vals_b, start, out, row0);
+                           (int)degree, p.keep, cap, best_slots, keys, start, out, row0);
     }
     VL_LAUNCH_CHECK("reverse_merge_kernel");
     return VL_OK;

@@ -74,11 +74,15 @@ def _workspace(device) -> _Workspace:
     return ws
 
 
-def release_workspaces() -> None:
+def release_workspaces(streams=None) -> None:
     """Drop the scratch memory kept for beam searches (one block per device and stream, sized by the largest
-    batch seen; several GB after a large build).  The next search allocates what it needs again."""
+    batch seen; several GB after a large build) - of the given torch streams only, or of all.  The next search
+    on such a stream allocates what it needs again."""
+    only = None if streams is None else {int(st.cuda_stream) for st in streams}
     with _WORKSPACES_LOCK:
-        for ws in _WORKSPACES.values():
+        for ((_, stream), ws) in _WORKSPACES.items():
+            if only is not None and stream not in only:
+                continue
             with ws.lock:
                 ws.tensor = None
 
@@ -302,6 +306,10 @@ class GraphBuild:
             if recall == 1.0:  # ann.py:187
                 break
         self.finished = True
+        if self._streams is not None:
+            # the side streams' beam-search workspaces (one per batch in flight, each with its own distance cache)
+            # are only worth keeping while batches run
+            release_workspaces(self._streams)
 
     def _in_flight(self, run_batch, starts, lanes: int, device):
         """Runs run_batch(start, stream) for every start with `lanes` of them in flight, yielding
@@ -574,7 +582,8 @@ class ANN:
             for _ in build.steps():
                 pass
             self.build_stats: list = build.stats
-            self._sketch = build.sketch
+            # the build's sketch (N x (16 * ceil(dim / 16) + 8) bytes) is let go with the build: searches
+            # run without one unless they ask (search(sketch=True) makes it again)
             (self.beams, self.distances) = build.result()
             if keep_queues:
                 width = build.beams.size(1)
