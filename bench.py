@@ -371,6 +371,11 @@ def main():
                     help="also sweep the other search settings (entry points, columns ranked, nodes visited per "
                          "iteration, progress-check cadence, stop): a few hundred searches; off by default")
     ap.add_argument("--no-tuned", action="store_true", help="accepted for older command lines; the sweep is off by default")
+    ap.add_argument("--search-runs", type=int, default=5, help="timed runs per search setting (the median is reported)")
+    ap.add_argument("--queues", default="10,16,32,64,96,128,192,256",
+                    help="search-queue lengths swept in this order (the sweep stops at the first that reaches recall@10 0.95)")
+    ap.add_argument("--no-reference-seeding", action="store_true",
+                    help="skip the search sweep with the reference's circulant seeds")
     ap.add_argument("--detail", default=None,
                     help="write everything measured (sweeps, per-loop tables, launches per phase) to this JSON file")
     ap.add_argument("--knn-only", action="store_true",
@@ -575,7 +580,7 @@ def main():
                                    frac=flops / t_knn / 1e12 / MFMA_FP32_PEAK, bound="mfma")
         log(f"[bench] exact kNN: {t_knn:.3f} s = {result['exact_knn']['tflops']:.1f} TFLOP/s")
 
-        def one_search(qs, seeding, mode, runs=5):
+        def one_search(qs, seeding, mode, runs=args.search_runs):
             """Median of `runs` whole searches of all queries, each between two HIP events on the launch stream
             (the search's own progress checks synchronise the host in between, as in any use of it)."""
             ann.search(qdev[:256].contiguous(), queue_size=qs, seeding=seeding, stop=mode)  # warm this shape
@@ -595,7 +600,7 @@ def main():
 
         def sweep_search(seeding, mode):
             sweep, chosen = [], None
-            for qs in (10, 16, 32, 64, 96, 128, 192, 256):
+            for qs in [int(x) for x in args.queues.split(",")]:
                 sweep.append(one_search(qs, seeding, mode))
                 if chosen is None and sweep[-1]["recall_at_10"] >= 0.95:
                     chosen = sweep[-1]
@@ -611,7 +616,8 @@ def main():
         # rows that are quiet stop expanding on their own (an addition; not bit-exact against the reference)
         result["search_per_query_stop"] = sweep_search("dense", "per_query")
         # the reference's query-independent circulant seeds, for comparison
-        result["search_reference_seeding"] = sweep_search("circulant", "batch")
+        if not args.no_reference_seeding:
+            result["search_reference_seeding"] = sweep_search("circulant", "batch")
         # roofline of the search iterations and of the seeding tiles at the reported queue length
         qs = result["search"]["queue"]
         profile_read(nv, reset=True, enable=1)
