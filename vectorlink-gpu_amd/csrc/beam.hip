@@ -472,8 +472,8 @@ __device__ __forceinline__ MergeResult merge_row(const MergeArgs &a, unsigned ch
     const int Pc = a.Pc;
     uint64_t *raw = reinterpret_cast<uint64_t *>(smem);  // candidate keys as they arrive
     uint64_t *uk = raw + Pc;                             // the candidates that can matter, then sorted
-    uint64_t *cc = RESIDENT ? raw : uk + Pc;             // filtered for one merge (raw is no longer needed by then)
-    uint64_t *qa = RESIDENT ? rr->qa : cc + Pc;          // search queue [0, L)
+    uint64_t *cc = raw;                                  // filtered for one merge (raw is no longer needed by then)
+    uint64_t *qa = RESIDENT ? rr->qa : uk + Pc;          // search queue [0, L)
     uint64_t *va = RESIDENT ? rr->va + a.Vt : qa + a.L;  // visit queue [Vt, VL)
     int32_t *seen_a = RESIDENT ? rr->seen_a : reinterpret_cast<int32_t *>(va + a.VL);
     int32_t *seen_b = RESIDENT ? rr->seen_b : seen_a + a.E;
@@ -876,7 +876,7 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
     }
     uint64_t *raw = reinterpret_cast<uint64_t *>(smem);
     uint64_t *uk = raw + a.Pc;
-    uint64_t *qa = uk + 2 * a.Pc;
+    uint64_t *qa = uk + a.Pc;
     uint64_t *va = qa + a.L;
     int32_t *seen_a = reinterpret_cast<int32_t *>(va + a.VL);
     int32_t *exl = seen_a + 2 * a.E;
@@ -901,14 +901,17 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
         probe_asked_s = 0;
     }
     // The neighbour lists of the nodes visited in one iteration share ids; only one copy of an id is evaluated.
-    // Every candidate claims its id in a hash set in LDS (the merge phase's array for filtered keys, free until
-    // then: 2 * Pc slots for at most m <= Pc ids, each the slot number of the claiming candidate); a candidate that
-    // finds its id claimed becomes the empty pair before anything is asked of memory for it.  The reference
-    // evaluates every copy (kernels.py:238-255) and drops all but one when the queues are sorted
-    // (kernels.py:314-349): copies carry the same distance, so what the queues receive is the same.
-    int32_t *const dset = reinterpret_cast<int32_t *>(uk + a.Pc);
-    const uint32_t dmask = 2u * (uint32_t)a.Pc - 1u;
-    for (int i = tid; i < 2 * a.Pc; i += THREADS) dset[i] = -1;
+    // Every candidate claims its id in a hash set in LDS (the second copy of the visited list, which the merge
+    // phase fills only later: E slots, each the slot number of the claiming candidate; used when that leaves the
+    // set at most two thirds full); a candidate that finds its id claimed becomes the empty pair before anything
+    // is asked of memory for it.  The reference evaluates every copy (kernels.py:238-255) and drops all but one
+    // when the queues are sorted (kernels.py:314-349): copies carry the same distance, so what the queues receive
+    // is the same.
+    int32_t *const dset = seen_a + a.E;
+    const uint32_t dsize = (uint32_t)a.E;
+    const bool dedup = 2 * a.E >= 3 * a.m;
+    if (dedup)
+        for (int i = tid; i < a.E; i += THREADS) dset[i] = -1;
     __syncthreads();
 
     // ---- expand: ann.py:69-73 (pop the visit heads, gather their neighbour lists, distances) ----
@@ -967,17 +970,16 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
         bool ok = has && id != VL_MAXINT && id >= 0 && (int64_t)id < s.n_vectors;
         if (s.count_evals || resample) n_wanted += __popcll(__ballot(ok));
         if (has) li[slot] = ok ? id : VL_MAXINT;  // (before the claim: a candidate that meets this one in the set reads it)
-        if (ok) {
-            uint32_t h = ((uint32_t)id * 2654435761u) >> 7;
+        if (ok && dedup) {
+            uint32_t h = __umulhi((uint32_t)id * 2654435761u, dsize);
             for (;;) {
-                h &= dmask;
                 const int owner = atomicCAS(&dset[h], -1, slot);
                 if (owner == -1) break;     // first of its id
                 if (li[owner] == id) {      // a copy: only the first is evaluated
                     ok = false;
                     break;
                 }
-                ++h;
+                h = h + 1 == dsize ? 0 : h + 1;
             }
             if (!ok) li[slot] = VL_MAXINT;
         }
@@ -1630,7 +1632,10 @@ void beam_window_sketch_kernel(StepArgs s) {
 // for.  The sketch's copy of the query row takes 16 registers per chunk and lane, and a row's phases (sketch
 // pass, two rounds of exact rows, merge) each wait on memory, so residency is worth a few spilled registers:
 // measured at 768 and 384 columns, five wavefronts per SIMD with two loads in flight beat three wavefronts
-// with four (0.84 -> 0.75 ms and 0.61 -> 0.43 ms per launch).
+// with four (0.84 -> 0.75 ms and 0.61 -> 0.43 ms per launch).  Residency is what a launch that is not bound by
+// memory traffic responds to (768 columns, state of the second optimisation loop, workgroups per compute unit
+// limited through LDS: 4 / 5 / 6 -> 0.53 / 0.46 / 0.42 ms per launch; 8 with one load in flight and 62 registers:
+// 0.415), which is also why the step's LDS arrays are overlaid where their lifetimes allow.
 template <int CPL, int LPR, int U, int THREADS, int SCPL, int SLPR, int SU, int WPE>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPE)))
 void beam_step_sketch_kernel(StepArgs s) {
@@ -1715,7 +1720,7 @@ int launch_step_by_dim(const StepArgs &s, bool aligned, int threads, size_t smem
     else if (nchunks <= 64) launch_step<1, 64, 8, false, 2, 8, 2, 5, 8, 6>(s, threads, smem, st);
     else if (nchunks <= 96 && variant != 1) launch_step<3, 32, 4, false, 3, 8, 2, 6, 2>(s, threads, smem, st);
     else if (nchunks <= 128) launch_step<2, 64, 8, false, 2, 16, 2, 6, 2>(s, threads, smem, st);
-    else if (nchunks <= 192) launch_step<3, 64, 4, false, 3, 16, 2, 5, 4, 6>(s, threads, smem, st);
+    else if (nchunks <= 192) launch_step<3, 64, 2, false, 3, 16, 1, 8, 1, 6>(s, threads, smem, st);
     else if (nchunks <= 256) launch_step<4, 64, 4, false, 4, 16, 2, 5, 2>(s, threads, smem, st);
     else if (nchunks <= 320) launch_step<5, 64, 2, false, 3, 32, 2, 6, 1>(s, threads, smem, st);
     else if (nchunks <= 384) launch_step<6, 64, 2, false, 3, 32, 2, 6, 1>(s, threads, smem, st);
@@ -1883,7 +1888,7 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
     const int Pmax = a.Ps > a.Pv ? a.Ps : a.Pv;
     const size_t smem = use_sort_merge
         ? (size_t)Pmax * 8 + (size_t)a.L * 4 + (size_t)a.E * 8 + (size_t)a.excl_cols * 4
-        : (size_t)a.Pc * 24 + (size_t)(a.L + a.VL) * 8 + (size_t)a.E * 8 + (size_t)a.excl_cols * 4 + (size_t)a.m + 16;
+        : (size_t)a.Pc * 16 + (size_t)(a.L + a.VL) * 8 + (size_t)a.E * 8 + (size_t)a.excl_cols * 4 + (size_t)a.m + 16;
     VL_REQUIRE(smem + 2048 <= kLdsPerCu, "queues of this size need %zu bytes of LDS (a compute unit has %zu)", smem,
                kLdsPerCu);
 
