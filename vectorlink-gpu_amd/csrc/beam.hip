@@ -465,7 +465,8 @@ struct MergeResult {
     bool queue_moved;  // RESIDENT: the search queue was written to qa_out (else it is unchanged in qa)
 };
 
-template <int THREADS, bool FUSED, class Refine = NoRefine, bool RESIDENT = false>
+// PREFILTERED: the caller has already dropped every candidate that the updated visited list holds.
+template <int THREADS, bool FUSED, class Refine = NoRefine, bool RESIDENT = false, bool PREFILTERED = false>
 __device__ __forceinline__ MergeResult merge_row(const MergeArgs &a, unsigned char *smem, RowState pre = RowState{0, 0},
                                                  Refine refine = Refine(), const ResidentRow *rr = nullptr) {
     static_assert(FUSED || !RESIDENT, "a resident row is a fused one");
@@ -619,7 +620,7 @@ __device__ __forceinline__ MergeResult merge_row(const MergeArgs &a, unsigned ch
         if (id != VL_MAXINT) {
             if (k < ws) f |= 1;
             if (!seen_full && k != wv) {  // k == wv is the visit queue's own last slot again
-                bool unseen = !sorted_contains(seen_b, cnt, id);
+                bool unseen = PREFILTERED || !sorted_contains(seen_b, cnt, id);
                 if (unseen) f |= (k < wv) ? 1 : 2;
             }
         }
@@ -724,7 +725,7 @@ __device__ __forceinline__ MergeResult merge_row(const MergeArgs &a, unsigned ch
         uint64_t k = uk[i];
         int32_t id = vl_key_id(k);
         if (i > 0 && id == vl_key_id(uk[i - 1])) return false;
-        if (sorted_contains(seen_b, cnt, id)) return false;      // kernels.py:471-488
+        if (!PREFILTERED && sorted_contains(seen_b, cnt, id)) return false;      // kernels.py:471-488
         int p = key_lower_bound(va, nva, k);
         return !(p < nva && va[p] == k);
     };
@@ -962,13 +963,27 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
     int n_wanted = 0, n_fetched = 0, n_sketched = 0;  // counts of this wavefront
     float *le = reinterpret_cast<float *>(raw);                     // upper bounds (raw is filled in the merge phase)
     uint8_t *xf = reinterpret_cast<uint8_t *>(exl + a.excl_cols);   // the merge phase's per-candidate flags; 16 = exact
-    // first pass over this wavefront's candidates: ids to LDS, later copies of an id out
+    // A candidate that the visited list holds once this iteration has updated it - an id visited earlier, or one
+    // popped now that the list still has room for (utils.py:73-75) - can change neither queue: the visit queue
+    // excludes it (ann.py:85-88), and the search queue met it with this very distance when it was first a candidate
+    // (every visited id came out of the visit queue, which is fed from the search queue's heads and then with the
+    // candidates the search queue is offered in the same iteration, ann.py:75-88), so it either still sits there
+    // or lies beyond its last slot, which only ever moves down.  Such candidates become the empty pair here,
+    // before a probe or a row is spent on them, and the merge phase knows the others to be unvisited.
+    const int n_popped_kept = pre.first >= a.E ? 0 : min(min(a.E - pre.first, a.Vt), a.E - pre.cnt);
+    __syncthreads();  // the visited list is in LDS
+    // first pass over this wavefront's candidates: ids to LDS, visited ids and later copies of an id out
     for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
         if (c0 != wave * kWave) id = resolve(c0);
         const int slot = c0 + lane;
         const bool has = slot < a.m;
         bool ok = has && id != VL_MAXINT && id >= 0 && (int64_t)id < s.n_vectors;
         if (s.count_evals || resample) n_wanted += __popcll(__ballot(ok));
+        if (ok) {
+            bool visited = sorted_contains(seen_a, pre.cnt, id);
+            for (int j = 0; j < n_popped_kept; ++j) visited |= g_visit_s[j] == id;
+            ok = !visited;
+        }
         if (has) li[slot] = ok ? id : VL_MAXINT;  // (before the claim: a candidate that meets this one in the set reads it)
         if (ok && dedup) {
             uint32_t h = __umulhi((uint32_t)id * 2654435761u, dsize);
@@ -1074,7 +1089,7 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
                 if (cid != VL_MAXINT) {
                     const float lo = ld[i];
                     bool need = !(lo > ws_d);
-                    if (!seen_full && !sorted_contains(seen_b, cnt, cid)) {
+                    if (!seen_full) {  // (every candidate left is unvisited)
                         if (!(lo > wv_d)) need = true;
                         else f |= 2;  // unvisited and certainly above the visit queue's last live slot
                     }
@@ -1168,9 +1183,9 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
                 __syncthreads();
             }
         };
-        merge_row<THREADS, true>(a, smem, pre, refine);
+        merge_row<THREADS, true, decltype(refine), false, true>(a, smem, pre, refine);
     } else {
-        merge_row<THREADS, true>(a, smem, pre);
+        merge_row<THREADS, true, NoRefine, false, true>(a, smem, pre);
     }
 }
 
