@@ -99,6 +99,12 @@ __device__ __forceinline__ void stage_operand(const float *const (&p)[4], int kt
     }
 }
 
+// every query's shared bound starts at infinity
+__global__ void knn_bound_init_kernel(uint32_t *__restrict__ q_bound, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        q_bound[i] = 0x7F800000u;
+}
+
 // squared lengths of rows, one wavefront per row (the L2 tiles add them to -2 q.v)
 __global__ __launch_bounds__(256) void row_norms_kernel(const float *__restrict__ rows, int64_t n, int dim,
                                                         float *__restrict__ out) {
@@ -126,7 +132,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                                                       int dim, int64_t strip_len, int n_strips,
                                                       int n_qblocks, int q_group, uint64_t *__restrict__ cand,
                                                       const float *__restrict__ q_norm,
-                                                      const float *__restrict__ v_norm) {
+                                                      const float *__restrict__ v_norm, uint32_t *__restrict__ q_bound) {
     // two buffers per operand as separate arrays: the compiler can then tell that the loads
     // landing in one buffer do not touch the one being read
     __shared__ __align__(16) float sV0[TILE];
@@ -178,6 +184,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // A value can only matter if it is not above the KK-th best seen so far for its query; the
     // two half-waves hold lists of the same queries, so each uses the tighter of the two bounds.
     float bound[2] = {__builtin_inff(), __builtin_inff()};
+    // The KK-th best of ANY list of a query bounds the query's KK-th best overall, so the lists of a query - in
+    // this workgroup's other wavefronts and in the workgroups that take the other strips - share the smallest of
+    // theirs through q_bound (distances are not negative: their bit patterns order like unsigned integers).  A
+    // wavefront publishes its bound when it is below the shared one it last read and picks the shared one up a
+    // tile later, so neither access is waited for; a value read late is merely a weaker bound.
+    uint32_t shared_bits[2] = {0x7F800000u, 0x7F800000u};
 
     const int half = lane >> 5;   // which k of an MFMA pair this lane feeds
     const int l32 = lane & 31;
@@ -312,8 +324,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         // value passes while the bound is 1 or more (distances are clamped to 1)
         float thr[2];
 #pragma unroll
-        for (int cb = 0; cb < 2; ++cb)
+        for (int cb = 0; cb < 2; ++cb) {
+            bound[cb] = fminf(bound[cb], __builtin_bit_cast(float, shared_bits[cb]));  // what the other lists had a tile ago
             thr[cb] = bound[cb] >= 1.0f ? -__builtin_inff() : fmaf(-2.0f, bound[cb], 1.0f) - 4e-7f;
+        }
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
             float vn[16];
@@ -353,7 +367,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
         for (int cb = 0; cb < 2; ++cb) {
             const float own = kd[cb][KK - 1];
-            bound[cb] = fminf(own, __shfl_xor(own, 32));
+            bound[cb] = fminf(fminf(own, __shfl_xor(own, 32)), bound[cb]);
+            const int64_t q = q0 + 64 * wc + 32 * cb + l32;
+            if (q < n_queries) {
+                if (half == 0 && bound[cb] < __builtin_bit_cast(float, shared_bits[cb]))  // better than what was there
+                    __hip_atomic_fetch_min(q_bound + q, __builtin_bit_cast(uint32_t, bound[cb]), __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+                shared_bits[cb] = __hip_atomic_load(q_bound + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
     }
 
@@ -434,7 +455,7 @@ struct KnnPlan {
     int n_strips;
     int64_t strip_len;
     int n_cand;
-    int64_t cand_bytes;  // per-lane candidate lists; the rows' squared lengths (L2) follow
+    int64_t cand_bytes;  // per-lane candidate lists; the queries' shared bounds and the rows' squared lengths (L2) follow
     int64_t bytes;
 };
 
@@ -468,7 +489,7 @@ int knn_plan(int64_t n_queries, int64_t n_vectors, int64_t dim, int64_t k, KnnPl
     p->list_len = list_length(k);
     p->n_cand = (int)(strips * LISTS_PER_STRIP * p->list_len);
     p->cand_bytes = (n_queries > 0 ? n_queries : 1) * (int64_t)p->n_cand * 8;
-    p->bytes = p->cand_bytes + ((n_queries + n_vectors) * 4 + 15) / 16 * 16;
+    p->bytes = p->cand_bytes + ((2 * n_queries + n_vectors) * 4 + 15) / 16 * 16;
     return VL_OK;
 }
 
@@ -512,8 +533,11 @@ VL_EXPORT int vl_knn_exact_metric(const float *queries, int64_t n_queries, const
     const int64_t blocks = (q_blocks * p.n_strips + 7) / 8 * 8;
     VL_REQUIRE(blocks <= kMaxBlocks * 4, "too many tiles for one call");
     const bool l2 = metric == VL_METRIC_L2;
-    float *q_norm = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + p.cand_bytes);
+    uint32_t *q_bound = reinterpret_cast<uint32_t *>(reinterpret_cast<char *>(workspace) + p.cand_bytes);
+    float *q_norm = reinterpret_cast<float *>(q_bound + n_queries);
     float *v_norm = q_norm + n_queries;
+    hipLaunchKernelGGL(knn_bound_init_kernel, dim3(vl_grid_for(n_queries, 256)), dim3(256), 0, st, q_bound, n_queries);
+    VL_LAUNCH_CHECK("knn_bound_init_kernel");
     if (l2) {
         VL_REQUIRE((n_vectors + 3) / 4 <= kMaxBlocks * 4, "too many vectors for one call");
         hipLaunchKernelGGL(row_norms_kernel, dim3((unsigned)((n_queries + 3) / 4)), dim3(256), 0, st, queries,
@@ -527,11 +551,11 @@ VL_EXPORT int vl_knn_exact_metric(const float *queries, int64_t n_queries, const
         if (l2)                                                                                               \
             hipLaunchKernelGGL((knn_tile_kernel<KK, true>), dim3((unsigned)blocks), dim3(256), 0, st, queries, \
                                n_queries, vectors, n_vectors, (int)dim, p.strip_len, p.n_strips, (int)q_blocks, \
-                               (int)q_group, cand, q_norm, v_norm);                                           \
+                               (int)q_group, cand, q_norm, v_norm, q_bound);                                  \
         else                                                                                                  \
             hipLaunchKernelGGL((knn_tile_kernel<KK, false>), dim3((unsigned)blocks), dim3(256), 0, st, queries, \
                                n_queries, vectors, n_vectors, (int)dim, p.strip_len, p.n_strips, (int)q_blocks, \
-                               (int)q_group, cand, nullptr, nullptr);                                         \
+                               (int)q_group, cand, nullptr, nullptr, q_bound);                                \
     } while (0)
     switch (p.list_len) {
         case 1: VL_KNN_LAUNCH(1); break;
