@@ -888,6 +888,7 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
     const float *q_row = s.queries + row * s.dim;
     uint64_t *memo_row = s.memo ? s.memo + ((uint64_t)row << (32 - s.memo_shift)) : nullptr;
     __shared__ int probe_hits_s, probe_asked_s;
+    __shared__ uint8_t sketch_order_s[SCPL > 0 ? THREADS : 4];  // wave_sketch: 64 bytes per wavefront
     const bool resample = memo_row && t == kMemoDecide;
     if (memo_row && memo_rate < s.memo_min_rate) memo_row = nullptr;
     bool sketching = false;
@@ -1030,7 +1031,7 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
                 }
                 if (s.count_evals || resample) n_sketched += __popcll(__ballot(ok));
                 wave_sketch<SCPL, SLPR, SU>(sq, s.sketch, s.sketch_tails, s.sketch_chunks, id, ok, ld + c0, le + c0,
-                                            memo_row, s.memo_shift);
+                                            sketch_order_s + wave * kWave, memo_row, s.memo_shift);
             }
             n_fetched = n_sketched;  // for the share of cache hits: what the cache did not answer
         }
@@ -1280,6 +1281,7 @@ __device__ __forceinline__ void beam_window_body(const StepArgs &s) {
     const uint8_t *const rounded_row0 = s.rounded_queries + row * s.rounded_query_bytes;
     uint64_t *const memo_table = s.memo ? s.memo + ((uint64_t)row << (32 - s.memo_shift)) : nullptr;
     __shared__ int probe_hits_s, probe_asked_s, quiet_s, memo_word_s;
+    __shared__ uint8_t sketch_order_s[SCPL > 0 ? THREADS : 4];  // wave_sketch: 64 bytes per wavefront
     int cur_q = 0, cur_v = 0, cur_s = 0;
     bool queue_dirty = false;
 
@@ -1436,7 +1438,7 @@ __device__ __forceinline__ void beam_window_body(const StepArgs &s) {
                     }
                     if (s.count_evals || resample) n_sketched += __popcll(__ballot(ok));
                     wave_sketch<SCPL, SLPR, SU>(sq, s.sketch, s.sketch_tails, s.sketch_chunks, id, ok, ld + c0, le + c0,
-                                                memo_row, s.memo_shift, lds);
+                                                sketch_order_s + wave * kWave, memo_row, s.memo_shift, lds);
                 }
                 n_fetched = n_sketched;  // for the share of cache hits: what the cache did not answer
             }

@@ -132,6 +132,7 @@ __global__ __launch_bounds__(256) void sketch_bounds_kernel(const uint8_t *__res
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     __shared__ float out_lo[256 / kWave][kWave], out_hi[256 / kWave][kWave];
+    __shared__ uint8_t order[256 / kWave][kWave];
     SketchQuery<SCPL> sq;
     sketch_query_load<SCPL, SLPR>(sq, rounded + row * rounded_bytes, chunks);
     for (int c0 = wave * kWave; c0 < m; c0 += 256) {
@@ -140,7 +141,7 @@ __global__ __launch_bounds__(256) void sketch_bounds_kernel(const uint8_t *__res
         const bool ok = slot < m && id != VL_MAXINT && id >= 0 && (int64_t)id < n_vectors;
         out_lo[wave][lane] = VL_MAXFLOAT;
         out_hi[wave][lane] = VL_MAXFLOAT;
-        wave_sketch<SCPL, SLPR, 2>(sq, table, tails, chunks, id, ok, out_lo[wave], out_hi[wave]);
+        wave_sketch<SCPL, SLPR, 2>(sq, table, tails, chunks, id, ok, out_lo[wave], out_hi[wave], order[wave]);
         // (the wavefront's own LDS writes and reads are in program order)
         if (slot < m) {
             lo[row * m + slot] = out_lo[wave][lane];

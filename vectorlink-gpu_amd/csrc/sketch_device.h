@@ -99,46 +99,43 @@ __device__ __forceinline__ void sketch_query_load(SketchQuery<SCPL> &sq, const u
 // One wavefront: lane j holds candidate id `my_id` (valid when `ok`); the bounds of its distance to
 // the query go to out_lo[j] and out_hi[j].  SLPR lanes share a sketch row (64 / SLPR rows per load
 // instruction), a lane holds SCPL of its 16-byte chunks, SU loads of a group are in flight at a time.
+// The loop over the rows does the integer sums only: the k-th candidate's lane is looked up in `order`
+// (64 bytes of LDS that belong to this wavefront, filled here), a group slot past the last candidate takes
+// the last one again (same addresses, same sum, nothing conditional in the loop), and a row's sum goes to
+// out_lo of its candidate.  What turns a sum into bounds - the row's tail, asked for before the loop - and
+// the cache entry are each lane's own work for its own candidate afterwards, once for the wavefront
+// instead of once per load.
 template <int SCPL, int SLPR, int SU>
 __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const uint8_t *__restrict__ table,
                                             const uint8_t *__restrict__ tails, int data_chunks, int32_t my_id, bool ok,
-                                            float *__restrict__ out_lo, float *__restrict__ out_hi,
+                                            float *out_lo, float *out_hi, uint8_t *order,
                                             uint64_t *memo_row = nullptr, int memo_shift = 0,
                                             LdsMemo lds = LdsMemo{nullptr, 0}) {
     constexpr int G = kWave / SLPR;
+    const uint64_t mask = __ballot(ok);
+    if (!mask) return;  // uniform over the wavefront
     const int lane = threadIdx.x & (kWave - 1);
     const int grp = lane / SLPR;
     const int lig = lane % SLPR;
-    uint64_t mask = __ballot(ok);
-    while (mask) {
-        int mysrc[SU];
-        int32_t ids[SU];
+    const int n = __popcll(mask);
+    uint2 tail = make_uint2(0u, 0u);
+    if (ok) {
+        tail = *reinterpret_cast<const uint2 *>(tails + (int64_t)my_id * kSketchTailBytes);
+        order[__builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u))] = (uint8_t)lane;
+    }
+    int chunk_at[SCPL];  // a chunk past the row's last one reads the last one again and meets zeros of the query
+#pragma unroll
+    for (int i = 0; i < SCPL; ++i) chunk_at[i] = min(lig + SLPR * i, data_chunks - 1);
+    for (int k0 = 0; k0 < n; k0 += G * SU) {
+        int src[SU];
         uint4 r[SU][SCPL];
-        uint2 tail[SU];
 #pragma unroll
         for (int u = 0; u < SU; ++u) {
-            int s = -1;
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-                int pick = -1;
-                if (mask) {
-                    pick = __builtin_ctzll(mask);
-                    mask &= mask - 1;
-                }
-                s = (grp == g) ? pick : s;
-            }
-            mysrc[u] = s;
-            const int32_t id = __shfl(my_id, s >= 0 ? s : 0);
-            ids[u] = id;
+            src[u] = order[min(k0 + u * G + grp, n - 1)];
+            const int32_t id = __shfl(my_id, src[u]);
             const uint4 *row = reinterpret_cast<const uint4 *>(table + (int64_t)id * data_chunks * 16);
 #pragma unroll
-            for (int i = 0; i < SCPL; ++i) {
-                const int c = lig + SLPR * i;
-                if (s >= 0 && c < data_chunks) r[u][i] = row[c];
-                else r[u][i] = make_uint4(0u, 0u, 0u, 0u);  // meets zeros of the query
-            }
-            if (s >= 0 && lig == 0) tail[u] = *reinterpret_cast<const uint2 *>(tails + (int64_t)id * kSketchTailBytes);
-            else tail[u] = make_uint2(0u, 0u);
+            for (int i = 0; i < SCPL; ++i) r[u][i] = row[chunk_at[i]];
         }
 #pragma unroll
         for (int u = 0; u < SU; ++u) {
@@ -154,23 +151,25 @@ __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const u
             }
             // a lane's two sums are below 2^24 (at most 64 elements of 127 * 127 each), so they convert exactly
             const float acc = fold_lanes<SLPR>(__builtin_fmaf(128.0f, (float)sh, (float)sl));
-            if (lig == 0 && mysrc[u] >= 0) {
-                const float scale = __builtin_bit_cast(float, tail[u].x);
-                const float resid = half_bits_as_float(tail[u].y & 0xffffu), norm = half_bits_as_float(tail[u].y >> 16);
-                const float s_hat = (scale * sq.qscale) * acc;
-                // 4e-6: the integer sums are exact, the float operations that combine them (one fused
-                // multiply-add per lane, up to six adds across lanes, two products) each round by 2^-24 of at most
-                // ||q^|| ||v^||
-                const float eps = (sq.norm2 * resid + (sq.qerr + 4e-6f * sq.norm2) * (norm + resid) + sq.exactc * norm) * 1.0001f + 2e-7f;
-                // a row with a bound of infinity (not finite, or longer than a half can say) met by a query of
-                // zeros gives 0 x infinity: no NaN leaves here for finite inputs, the widest bounds do
-                const bool known = eps == eps;
-                const float lo = known ? clamp_distance(s_hat + eps) : 0.0f, hi = known ? clamp_distance(s_hat - eps) : 1.0f;
-                out_lo[mysrc[u]] = lo;
-                out_hi[mysrc[u]] = hi;
-                if (memo_row) memo_store_bounds(memo_row, memo_shift, ids[u], lo, hi);
-                if (lds.tab) lds_memo_store(lds, ids[u], memo_bounds_entry(ids[u], lo, hi));
-            }
+            if (lig == 0) out_lo[src[u]] = acc;
         }
+    }
+    if (ok) {
+        const float acc = out_lo[lane];  // written by the first lane of the group that had this candidate's row
+        const float scale = __builtin_bit_cast(float, tail.x);
+        const float resid = half_bits_as_float(tail.y & 0xffffu), norm = half_bits_as_float(tail.y >> 16);
+        const float s_hat = (scale * sq.qscale) * acc;
+        // 4e-6: the integer sums are exact, the float operations that combine them (one fused
+        // multiply-add per lane, up to six adds across lanes, two products) each round by 2^-24 of at most
+        // ||q^|| ||v^||
+        const float eps = (sq.norm2 * resid + (sq.qerr + 4e-6f * sq.norm2) * (norm + resid) + sq.exactc * norm) * 1.0001f + 2e-7f;
+        // a row with a bound of infinity (not finite, or longer than a half can say) met by a query of
+        // zeros gives 0 x infinity: no NaN leaves here for finite inputs, the widest bounds do
+        const bool known = eps == eps;
+        const float lo = known ? clamp_distance(s_hat + eps) : 0.0f, hi = known ? clamp_distance(s_hat - eps) : 1.0f;
+        out_lo[lane] = lo;
+        out_hi[lane] = hi;
+        if (memo_row) memo_store_bounds(memo_row, memo_shift, my_id, lo, hi);
+        if (lds.tab) lds_memo_store(lds, my_id, memo_bounds_entry(my_id, lo, hi));
     }
 }
