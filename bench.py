@@ -311,6 +311,8 @@ def headline(result):
         out["scope"] = "algorithmic bytes / published HBM peak; served beyond L2"
         out.update(_pick(rf, ("avg_launch_ms", "algorithmic_bytes_per_launch", "launches_in_timed_build",
                               "copy_gbs_measured")))
+        if rf.get("in_timed_build"):
+            out["in_timed_build"] = _pick(rf["in_timed_build"], ("achieved", "frac", "batches_in_flight"), 3)
         if rf.get("gather_gbs_measured"):
             out["gather_gbs_measured"] = {k: _r(v, 3) for k, v in rf["gather_gbs_measured"].items()}
         out["per_loop"] = [_pick(r, ("loop", "avg_launch_ms", "algorithmic_bytes_per_launch", "frac",
@@ -544,6 +546,13 @@ def main():
         gather_gbs_measured=gather_gbs,
         avg_launch_ms=w_time / w_launch, algorithmic_bytes_per_launch=w_bytes / w_launch,
         launches_in_timed_build=int(sum(weights)),
+        # the same bytes over the wall time of the timed build's loops (everything a loop does included): with
+        # several batches in flight one batch's launch runs on the compute units that the last workgroups of
+        # another's leave idle, which a launch timed alone cannot show
+        in_timed_build=dict(achieved=w_bytes / max(sum(st["seconds"] for st in build.stats[:len(per_loop)]), 1e-9) / 1e9,
+                            frac=w_bytes / max(sum(st["seconds"] for st in build.stats[:len(per_loop)]), 1e-9) / 1e9
+                                 / HBM_PEAK_GBS,
+                            batches_in_flight=args.concurrent_batches),
         method=f"hooks are off in the timed build; the first {replay} batches of the tables each optimisation loop "
                "started from were run again with HIP events around the launches (on the launch stream) and the fetched "
                "rows counted on the device; per-loop averages below, combined here with the timed build's launch counts",
