@@ -349,48 +349,6 @@ __device__ inline void raise_running_max(int *slot, int cnt, int bound) {
     else atomicMax(slot, cnt);
 }
 
-// Smallest key over the workgroup of each thread's `mine` (kPadKey = none).
-// red: 2 * kQueueWaves keys of LDS, used alternately so one barrier per call suffices.
-__device__ inline uint64_t block_min_key(uint64_t mine, uint64_t *red, int round) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
-    const int nw = blockDim.x / kWave;
-    {
-        // folded like wave_min_u32 below, both words of a key moving together; lane 0 ends with the minimum
-        uint32_t lo = (uint32_t)mine, hi = (uint32_t)(mine >> 32);
-        auto take = [&](uint32_t olo, uint32_t ohi) {
-            const bool less = ohi < hi || (ohi == hi && olo < lo);
-            lo = less ? olo : lo;
-            hi = less ? ohi : hi;
-        };
-        {
-            uint32_t a0 = lo, a1 = lo, b0 = hi, b1 = hi;
-            asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\tv_permlane32_swap_b32 %2, %3\n\ts_nop 1"
-                         : "+v"(a0), "+v"(a1), "+v"(b0), "+v"(b1));
-            lo = a0; hi = b0;
-            take(a1, b1);
-        }
-        {
-            uint32_t a0 = lo, a1 = lo, b0 = hi, b1 = hi;
-            asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\tv_permlane16_swap_b32 %2, %3\n\ts_nop 1"
-                         : "+v"(a0), "+v"(a1), "+v"(b0), "+v"(b1));
-            lo = a0; hi = b0;
-            take(a1, b1);
-        }
-        take(__builtin_amdgcn_update_dpp(lo, lo, 0x108, 0xf, 0xf, false), __builtin_amdgcn_update_dpp(hi, hi, 0x108, 0xf, 0xf, false));
-        take(__builtin_amdgcn_update_dpp(lo, lo, 0x104, 0xf, 0xf, false), __builtin_amdgcn_update_dpp(hi, hi, 0x104, 0xf, 0xf, false));
-        take(__builtin_amdgcn_update_dpp(lo, lo, 0x102, 0xf, 0xf, false), __builtin_amdgcn_update_dpp(hi, hi, 0x102, 0xf, 0xf, false));
-        take(__builtin_amdgcn_update_dpp(lo, lo, 0x101, 0xf, 0xf, false), __builtin_amdgcn_update_dpp(hi, hi, 0x101, 0xf, 0xf, false));
-        mine = ((uint64_t)hi << 32) | lo;
-    }
-    uint64_t *slot = red + (round & 1) * kQueueWaves;
-    if (lane == 0) slot[wave] = mine;
-    __syncthreads();
-    uint64_t m = slot[0];
-    for (int w = 1; w < nw; ++w) m = slot[w] < m ? slot[w] : m;
-    return m;
-}
-
 // Smallest 32-bit value over a wavefront, in every lane: halves and rows are folded with the swap instructions
 // and DPP row shifts that fold_group uses (a lane without a source keeps its own value), a few cycles per
 // step where a cross-lane shuffle through the LDS crossbar takes a round trip each.
@@ -426,6 +384,15 @@ __device__ inline uint32_t block_min_u32(uint32_t mine, uint32_t *red, int round
     uint32_t m = slot[0];
     for (int w = 1; w < nw; ++w) m = slot[w] < m ? slot[w] : m;
     return m;
+}
+
+// A candidate's upper bound (a cosine distance, in [0, 1]) and its slot in one 32-bit key, smallest bound first:
+// the bound to 19 bits, rounded down, then the slot (a row has at most kMaxCandidates candidate slots: more would
+// not fit the LDS).  Only used to choose which candidates to look at first - any choice is a valid one there - so
+// the rounding costs nothing but a slightly different pick among near-equal bounds.  Never 0xFFFFFFFF.
+constexpr int kMaxCandidates = 8192;
+__device__ __forceinline__ uint32_t bound_slot_key(float hi, int slot) {
+    return ((uint32_t)(hi * 524286.0f) << 13) | (uint32_t)slot;
 }
 
 // Workgroup-wide scalars shared by the expand and merge phases of a row.
@@ -888,7 +855,7 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
     const float *q_row = s.queries + row * s.dim;
     uint64_t *memo_row = s.memo ? s.memo + ((uint64_t)row << (32 - s.memo_shift)) : nullptr;
     __shared__ int probe_hits_s, probe_asked_s;
-    __shared__ uint8_t sketch_order_s[SCPL > 0 ? THREADS : 4];  // wave_sketch: 64 bytes per wavefront
+    __shared__ uint8_t lane_order_s[THREADS];  // wave_sketch, wave_distances_lds: 64 bytes per wavefront
     const bool resample = memo_row && t == kMemoDecide;
     if (memo_row && memo_rate < s.memo_min_rate) memo_row = nullptr;
     bool sketching = false;
@@ -1031,7 +998,7 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
                 }
                 if (s.count_evals || resample) n_sketched += __popcll(__ballot(ok));
                 wave_sketch<SCPL, SLPR, SU>(sq, s.sketch, s.sketch_tails, s.sketch_chunks, id, ok, ld + c0, le + c0,
-                                            sketch_order_s + wave * kWave, memo_row, s.memo_shift);
+                                            lane_order_s + wave * kWave, memo_row, s.memo_shift);
             }
             n_fetched = n_sketched;  // for the share of cache hits: what the cache did not answer
         }
@@ -1052,7 +1019,8 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
         if constexpr (GENERIC)
             wave_distances_generic(q_row, s.vectors, s.dim, s.nchunks, id, ok, ld + c0, memo_row, s.memo_shift, s.l2 != 0);
         else
-            wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, id, ok, ld + c0, memo_row, s.memo_shift, s.l2 != 0);
+            wave_distances_lds<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, id, ok, ld + c0, lane_order_s + wave * kWave,
+                                            memo_row, s.memo_shift, s.l2 != 0);
     }
     if (s.count_evals && lane == 0) {
         const int stripe = (int)((blockIdx.x * (THREADS / kWave) + wave) & (kBeamStripes - 1));
@@ -1105,18 +1073,18 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
             bool all_rest = false;
             if (!seen_full) {
                 for (int r = 0; r < a.Vt; ++r) {
-                    uint64_t mine = kPadKey;
+                    uint32_t mine = 0xFFFFFFFFu;
                     for (int i = tid; i < a.m; i += THREADS) {
                         if ((flags[i] & (2 | 8)) != 2) continue;
-                        const uint64_t k = vl_make_key(li[i], le[i]);
+                        const uint32_t k = bound_slot_key(le[i], i);
                         if (k < mine) mine = k;
                     }
-                    const uint64_t mn = block_min_key(mine, red, r);
-                    if (mn == kPadKey) {
+                    const uint32_t mn = block_min_u32(mine, reinterpret_cast<uint32_t *>(red), r);
+                    if (mn == 0xFFFFFFFFu) {
                         all_rest = true;
                         break;
                     }
-                    const int32_t chosen = vl_key_id(mn);
+                    const int32_t chosen = li[mn & (kMaxCandidates - 1)];
                     for (int i = tid; i < a.m; i += THREADS)
                         if ((flags[i] & 2) && li[i] == chosen) flags[i] |= 8;
                 }
@@ -1132,21 +1100,22 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
                 if (ok) flags[slot] = f | 16;  // its distance is exact from here on
                 n_exact += __popcll(__ballot(ok));
                 n_real += __popcll(__ballot(cid != VL_MAXINT && !(f & 16)));  // candidates known by bounds only
-                wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0, memo_row, s.memo_shift, false);
+                wave_distances_lds<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0,
+                                                lane_order_s + wave * kWave, memo_row, s.memo_shift, false);
             }
             __syncthreads();
             // tv: the largest exact distance of those Vt candidates.  Vt distinct unvisited candidates above wv
             // are at most tv, so a candidate whose lower bound is above tv is not one of the Vt smallest.
             float tv = -1.0f;
             if (!seen_full && !all_rest) {
-                uint64_t mine = kPadKey;
+                uint32_t mine = 0xFFFFFFFFu;  // (no distance has the key 0)
                 for (int i = tid; i < a.m; i += THREADS)
                     if (flags[i] & 8) {
-                        const uint64_t k = ~(uint64_t)vl_float_key(ld[i]);
+                        const uint32_t k = ~vl_float_key(ld[i]);
                         mine = k < mine ? k : mine;
                     }
-                const uint64_t mn = block_min_key(mine, red, a.Vt);
-                tv = mn == kPadKey ? -1.0f : vl_key_float((uint32_t)~mn);
+                const uint32_t mn = block_min_u32(mine, reinterpret_cast<uint32_t *>(red), a.Vt);
+                tv = mn == 0xFFFFFFFFu ? -1.0f : vl_key_float(~mn);
             }
             // second round: the candidates above wv that may still be among the Vt smallest
             for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
@@ -1160,7 +1129,8 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
                     ld[slot] = VL_MAXFLOAT;
                 }
                 n_exact += __popcll(__ballot(ok));
-                wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0, memo_row, s.memo_shift, false);
+                wave_distances_lds<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0,
+                                                lane_order_s + wave * kWave, memo_row, s.memo_shift, false);
             }
             if (s.count_evals && lane == 0 && n_exact)
                 atomicAdd(&c->evals[(int)((blockIdx.x * (THREADS / kWave) + wave) & (kBeamStripes - 1))],
@@ -1281,7 +1251,7 @@ __device__ __forceinline__ void beam_window_body(const StepArgs &s) {
     const uint8_t *const rounded_row0 = s.rounded_queries + row * s.rounded_query_bytes;
     uint64_t *const memo_table = s.memo ? s.memo + ((uint64_t)row << (32 - s.memo_shift)) : nullptr;
     __shared__ int probe_hits_s, probe_asked_s, quiet_s, memo_word_s;
-    __shared__ uint8_t sketch_order_s[SCPL > 0 ? THREADS : 4];  // wave_sketch: 64 bytes per wavefront
+    __shared__ uint8_t lane_order_s[THREADS];  // wave_sketch, wave_distances_lds: 64 bytes per wavefront
     int cur_q = 0, cur_v = 0, cur_s = 0;
     bool queue_dirty = false;
 
@@ -1438,7 +1408,7 @@ __device__ __forceinline__ void beam_window_body(const StepArgs &s) {
                     }
                     if (s.count_evals || resample) n_sketched += __popcll(__ballot(ok));
                     wave_sketch<SCPL, SLPR, SU>(sq, s.sketch, s.sketch_tails, s.sketch_chunks, id, ok, ld + c0, le + c0,
-                                                sketch_order_s + wave * kWave, memo_row, s.memo_shift, lds);
+                                                lane_order_s + wave * kWave, memo_row, s.memo_shift, lds);
                 }
                 n_fetched = n_sketched;  // for the share of cache hits: what the cache did not answer
             }
@@ -1461,8 +1431,8 @@ __device__ __forceinline__ void beam_window_body(const StepArgs &s) {
                 }
             }
             if (s.count_evals || resample) n_fetched += __popcll(__ballot(ok));
-            wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, id, ok, ld + c0, memo_row, s.memo_shift,
-                                        s.l2 != 0, lds);
+            wave_distances_lds<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, id, ok, ld + c0, lane_order_s + wave * kWave,
+                                            memo_row, s.memo_shift, s.l2 != 0, lds);
         }
         if (s.count_evals && lane == 0) {
             const int stripe = (int)((blockIdx.x * (THREADS / kWave) + wave) & (kBeamStripes - 1));
@@ -1512,18 +1482,18 @@ __device__ __forceinline__ void beam_window_body(const StepArgs &s) {
                 bool all_rest = false;
                 if (!seen_full) {
                     for (int r = 0; r < a.Vt; ++r) {
-                        uint64_t mine = kPadKey;
+                        uint32_t mine = 0xFFFFFFFFu;
                         for (int i = tid; i < a.m; i += THREADS) {
                             if ((flags[i] & (2 | 8)) != 2) continue;
-                            const uint64_t k = vl_make_key(li[i], le[i]);
+                            const uint32_t k = bound_slot_key(le[i], i);
                             if (k < mine) mine = k;
                         }
-                        const uint64_t mn = block_min_key(mine, red, r);
-                        if (mn == kPadKey) {
+                        const uint32_t mn = block_min_u32(mine, reinterpret_cast<uint32_t *>(red), r);
+                        if (mn == 0xFFFFFFFFu) {
                             all_rest = true;
                             break;
                         }
-                        const int32_t chosen = vl_key_id(mn);
+                        const int32_t chosen = li[mn & (kMaxCandidates - 1)];
                         for (int i = tid; i < a.m; i += THREADS)
                             if ((flags[i] & 2) && li[i] == chosen) flags[i] |= 8;
                     }
@@ -1538,20 +1508,20 @@ __device__ __forceinline__ void beam_window_body(const StepArgs &s) {
                     if (ok) flags[slot] = f | 16;
                     n_exact += __popcll(__ballot(ok));
                     n_real += __popcll(__ballot(cid != VL_MAXINT && !(f & 16)));
-                    wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0, memo_row, s.memo_shift,
-                                                false, lds);
+                    wave_distances_lds<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0,
+                                                    lane_order_s + wave * kWave, memo_row, s.memo_shift, false, lds);
                 }
                 __syncthreads();
                 float tv = -1.0f;
                 if (!seen_full && !all_rest) {
-                    uint64_t mine = kPadKey;
+                    uint32_t mine = 0xFFFFFFFFu;  // (no distance has the key 0)
                     for (int i = tid; i < a.m; i += THREADS)
                         if (flags[i] & 8) {
-                            const uint64_t k = ~(uint64_t)vl_float_key(ld[i]);
+                            const uint32_t k = ~vl_float_key(ld[i]);
                             mine = k < mine ? k : mine;
                         }
-                    const uint64_t mn = block_min_key(mine, red, a.Vt);
-                    tv = mn == kPadKey ? -1.0f : vl_key_float((uint32_t)~mn);
+                    const uint32_t mn = block_min_u32(mine, reinterpret_cast<uint32_t *>(red), a.Vt);
+                    tv = mn == 0xFFFFFFFFu ? -1.0f : vl_key_float(~mn);
                 }
                 for (int c0 = wave * kWave; c0 < a.m; c0 += THREADS) {
                     const int slot = c0 + lane;
@@ -1564,8 +1534,8 @@ __device__ __forceinline__ void beam_window_body(const StepArgs &s) {
                         ld[slot] = VL_MAXFLOAT;
                     }
                     n_exact += __popcll(__ballot(ok));
-                    wave_distances<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0, memo_row, s.memo_shift,
-                                                false, lds);
+                    wave_distances_lds<CPL, LPR, U>(q_row, s.vectors, s.dim, s.nchunks, cid, ok, ld + c0,
+                                                    lane_order_s + wave * kWave, memo_row, s.memo_shift, false, lds);
                 }
                 if (s.count_evals && lane == 0 && n_exact)
                     atomicAdd(&c->evals[(int)((blockIdx.x * (THREADS / kWave) + wave) & (kBeamStripes - 1))],
@@ -1940,7 +1910,7 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
         step.memo_min_rate = rate_env >= 0 ? rate_env : (int)(r > 255 ? 255 : r);
     }
     // The sketch serves the cosine distance of 16-byte aligned rows in the fused step; other calls ignore it.
-    step.sketch = (sketch && !step.l2 && aligned && use_fused && p->dim <= 2048) ? sketch : nullptr;
+    step.sketch = (sketch && !step.l2 && aligned && use_fused && p->dim <= 2048 && l.m <= kMaxCandidates) ? sketch : nullptr;
     VL_REQUIRE(!step.sketch || (p->flags & VL_BEAM_USES_SKETCH),
                "a call with a sketch needs VL_BEAM_USES_SKETCH in flags (and a workspace sized with it)");
     step.rounded_queries = (const uint8_t *)(ws + l.off_rounded);

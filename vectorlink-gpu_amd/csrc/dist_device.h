@@ -212,6 +212,109 @@ __device__ __forceinline__ void wave_distances(const float *__restrict__ q_row,
     }
 }
 
+// The same distances for a caller whose out_d is in LDS (the fused beam-search step), with the per-row work cut to
+// the sums: the k-th candidate's lane comes from `order` (64 bytes of LDS that belong to this wavefront, filled
+// here by rank; with one row per load instruction the lanes are simply taken off the mask), a group slot past the last
+// candidate takes the last one again (same addresses, same sum: nothing in the loop depends on a lane having a
+// row), and the group's first lane parks the row's sum in out_d of its candidate.  Turning a sum into a distance
+// and storing the cache entry is then each lane's own work for its own candidate, once for the wavefront instead
+// of once per load.  Same loads, same additions in the same order, same bits as wave_distances.
+template <int CPL, int LPR, int U>
+__device__ __forceinline__ void wave_distances_lds(const float *__restrict__ q_row,
+                                                   const float *__restrict__ vectors, int dim,
+                                                   int nchunks, int32_t my_id, bool ok,
+                                                   float *out_d, uint8_t *order, uint64_t *memo_row,
+                                                   int memo_shift, bool l2 = false, LdsMemo lds = LdsMemo{nullptr, 0}) {
+    constexpr int G = kWave / LPR;
+    uint64_t mask = __ballot(ok);
+    if (!mask) return;  // uniform over the wavefront
+    const int lane = threadIdx.x & (kWave - 1);
+    const int grp = lane / LPR;
+    const int lig = lane % LPR;
+    const int n = __popcll(mask);
+
+    float4 q[CPL];
+    bool cvalid[CPL];
+#pragma unroll
+    for (int i = 0; i < CPL; ++i) {
+        int c = lig + LPR * i;
+        cvalid[i] = c < nchunks;
+        q[i] = cvalid[i] ? reinterpret_cast<const float4 *>(q_row)[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if constexpr (G > 1) {
+        if (ok) order[__builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u))] = (uint8_t)lane;
+    }
+    for (int k0 = 0; k0 < n; k0 += G * U) {
+        float4 r[U][CPL];
+        int src[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (k0 + u * G < n) {  // uniform: a load instruction with no candidate at all is not issued
+                int32_t id;
+                if constexpr (G == 1) {
+                    src[u] = __builtin_ctzll(mask);
+                    mask &= mask - 1;
+                    id = __builtin_amdgcn_readlane(my_id, src[u]);
+                } else {
+                    src[u] = order[min(k0 + u * G + grp, n - 1)];
+                    id = __shfl(my_id, src[u]);
+                }
+                const float4 *row = reinterpret_cast<const float4 *>(vectors + (int64_t)id * dim);
+#pragma unroll
+                for (int i = 0; i < CPL; ++i) {
+                    if (cvalid[i]) r[u][i] = row[lig + LPR * i];
+                    else r[u][i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (k0 + u * G < n) {
+                // the partial sums of wave_distances, folded in the same order
+                constexpr int V = kWave / LPR;
+                float part[V];
+#pragma unroll
+                for (int j = 0; j < V; ++j) part[j] = 0.0f;
+                if (l2) {  // uniform over the launch
+#pragma unroll
+                    for (int i = 0; i < CPL; ++i) {
+                        const float dx = r[u][i].x - q[i].x, dy = r[u][i].y - q[i].y;
+                        const float dz = r[u][i].z - q[i].z, dw = r[u][i].w - q[i].w;
+                        float a = part[i % V];
+                        a = __builtin_fmaf(dx, dx, a);
+                        a = __builtin_fmaf(dy, dy, a);
+                        a = __builtin_fmaf(dz, dz, a);
+                        a = __builtin_fmaf(dw, dw, a);
+                        part[i % V] = a;
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < CPL; ++i) {
+                        float a = part[i % V];
+                        a = __builtin_fmaf(r[u][i].x, q[i].x, a);
+                        a = __builtin_fmaf(r[u][i].y, q[i].y, a);
+                        a = __builtin_fmaf(r[u][i].z, q[i].z, a);
+                        a = __builtin_fmaf(r[u][i].w, q[i].w, a);
+                        part[i % V] = a;
+                    }
+                }
+#pragma unroll
+                for (int h = V / 2; h >= 1; h >>= 1)
+#pragma unroll
+                    for (int j = 0; j < h; ++j) part[j] = part[j] + part[j + h];
+                const float acc = fold_group<LPR>(part[0]);
+                if (lig == 0) out_d[src[u]] = acc;
+            }
+        }
+    }
+    if (ok) {
+        const float d = finish_distance(out_d[lane], l2);  // the sum was parked there by the first lane of the row's group
+        out_d[lane] = d;
+        if (memo_row) memo_store(memo_row, memo_shift, my_id, d);
+        if (lds.tab) lds_memo_store(lds, my_id, memo_entry(my_id, d));
+    }
+}
+
 // Any dimension, any alignment: scalar loads, same summation order.
 __device__ __forceinline__ void wave_distances_generic(const float *__restrict__ q_row,
                                                        const float *__restrict__ vectors, int dim,

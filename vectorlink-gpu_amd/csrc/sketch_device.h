@@ -131,6 +131,7 @@ __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const u
         uint4 r[SU][SCPL];
 #pragma unroll
         for (int u = 0; u < SU; ++u) {
+            if (k0 + u * G >= n) continue;  // uniform: a load instruction with no candidate at all is not issued
             src[u] = order[min(k0 + u * G + grp, n - 1)];
             const int32_t id = __shfl(my_id, src[u]);
             const uint4 *row = reinterpret_cast<const uint4 *>(table + (int64_t)id * data_chunks * 16);
@@ -139,6 +140,7 @@ __device__ __forceinline__ void wave_sketch(const SketchQuery<SCPL> &sq, const u
         }
 #pragma unroll
         for (int u = 0; u < SU; ++u) {
+            if (k0 + u * G >= n) continue;
             int sh = 0, sl = 0;
 #pragma unroll
             for (int i = 0; i < SCPL; ++i) {
