@@ -398,6 +398,12 @@ __device__ __forceinline__ uint32_t bound_slot_key(float hi, int slot) {
 // Workgroup-wide scalars shared by the expand and merge phases of a row.
 __shared__ int g_n_ex_s;                  // exclusion ids before the row's first empty one
 __shared__ int32_t g_visit_s[kMaxVisit];  // the ids popped from the visit queue in this iteration
+// The ids the merge phase adds to the visited list (between two of its barriers).  The expand phase and the exact
+// rounds of a sketched row, which run before and after that, use the same 256 bytes as the wavefronts' lists of
+// candidate lanes (wave_sketch, wave_distances_lds: 64 bytes each) - sixteen 128-thread workgroups of the
+// 128-column shape fit a compute unit's LDS with these bytes shared and fifteen without.
+__shared__ int32_t g_new_s[kMaxVisit];
+static_assert(kMaxVisit * 4 >= 256, "one byte per thread of the largest workgroup");
 
 // What the fused step has read of a row before its merge phase starts.
 struct RowState {
@@ -449,7 +455,7 @@ __device__ __forceinline__ MergeResult merge_row(const MergeArgs &a, unsigned ch
     uint8_t *fl = RESIDENT ? rr->fl : reinterpret_cast<uint8_t *>(exl + a.excl_cols);  // per candidate: bit0 wanted, bit1 rest
     __shared__ int wave_cnt[kQueueWaves];
     __shared__ uint64_t red[2 * kQueueWaves];
-    __shared__ int32_t newv[kMaxVisit];
+    int32_t *const newv = g_new_s;
     __shared__ int n_new_s;
     __shared__ int row_changed_s;  // per-query stop: some slot of the search queue's first L changed
     int &n_ex_s = g_n_ex_s;
@@ -855,7 +861,7 @@ __device__ __forceinline__ void beam_step_body(const StepArgs &s) {
     const float *q_row = s.queries + row * s.dim;
     uint64_t *memo_row = s.memo ? s.memo + ((uint64_t)row << (32 - s.memo_shift)) : nullptr;
     __shared__ int probe_hits_s, probe_asked_s;
-    __shared__ uint8_t lane_order_s[THREADS];  // wave_sketch, wave_distances_lds: 64 bytes per wavefront
+    uint8_t *const lane_order_s = reinterpret_cast<uint8_t *>(g_new_s);  // 64 bytes per wavefront (see g_new_s)
     const bool resample = memo_row && t == kMemoDecide;
     if (memo_row && memo_rate < s.memo_min_rate) memo_row = nullptr;
     bool sketching = false;
@@ -1164,6 +1170,14 @@ template <int CPL, int LPR, int U, bool GENERIC, int THREADS>
 __global__ __launch_bounds__(THREADS) void beam_step_kernel(StepArgs s) {
     beam_step_body<CPL, LPR, U, GENERIC, THREADS>(s);
 }
+// The same kernel built to leave room for WPP wavefronts per SIMD.  Its vector registers would allow that anyway;
+// what does not is its scalar registers (more than 96 of them mean seven wavefronts instead of eight), which the
+// compiler keeps within bounds when asked, at the price of a few moves to and from lanes of a vector register.
+template <int CPL, int LPR, int U, int THREADS, int WPP>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPP)))
+void beam_step_kernel_w(StepArgs s) {
+    beam_step_body<CPL, LPR, U, false, THREADS>(s);
+}
 
 // ---- several iterations per launch ----------------------------------------------
 // While parallel_visit_count * t <= E (the visited list's width) no row's visited list can be full at
@@ -1251,7 +1265,7 @@ __device__ __forceinline__ void beam_window_body(const StepArgs &s) {
     const uint8_t *const rounded_row0 = s.rounded_queries + row * s.rounded_query_bytes;
     uint64_t *const memo_table = s.memo ? s.memo + ((uint64_t)row << (32 - s.memo_shift)) : nullptr;
     __shared__ int probe_hits_s, probe_asked_s, quiet_s, memo_word_s;
-    __shared__ uint8_t lane_order_s[THREADS];  // wave_sketch, wave_distances_lds: 64 bytes per wavefront
+    uint8_t *const lane_order_s = reinterpret_cast<uint8_t *>(g_new_s);  // 64 bytes per wavefront (see g_new_s)
     int cur_q = 0, cur_v = 0, cur_s = 0;
     bool queue_dirty = false;
 
@@ -1630,11 +1644,11 @@ void beam_step_sketch_kernel(StepArgs s) {
 }
 
 template <int CPL, int LPR, int U, bool GENERIC, int SCPL = 0, int SLPR = 64, int SU = 1, int WPE = 4, int UX = U,
-          int WPW = WPE>
+          int WPW = WPE, int WPP = 0>
 void launch_step(const StepArgs &s, int threads, size_t smem, hipStream_t st) {
     dim3 grid((unsigned)s.m.n_rows);
     if constexpr (SCPL > 0) {
-        if (!s.sketch) return launch_step<CPL, LPR, U, GENERIC, 0, 64, 1, WPE, U, WPW>(s, threads, smem, st);
+        if (!s.sketch) return launch_step<CPL, LPR, U, GENERIC, 0, 64, 1, WPE, U, WPW, WPP>(s, threads, smem, st);
     }
     if constexpr (!GENERIC) {
         if (s.window > 0) {  // several iterations in this launch (smem is the window kernel's size)
@@ -1670,6 +1684,16 @@ void launch_step(const StepArgs &s, int threads, size_t smem, hipStream_t st) {
             if (vl_allow_lds(kernel, smem) != hipSuccess) return;
             hipLaunchKernelGGL(kernel, grid, dim3(256), smem, st, s);
         }
+    } else if constexpr (WPP > 0 && !GENERIC) {
+        if (threads == 128) {
+            auto kernel = beam_step_kernel_w<CPL, LPR, U, 128, WPP>;
+            if (vl_allow_lds(kernel, smem) != hipSuccess) return;
+            hipLaunchKernelGGL(kernel, grid, dim3(128), smem, st, s);
+        } else {
+            auto kernel = beam_step_kernel_w<CPL, LPR, U, 256, WPP>;
+            if (vl_allow_lds(kernel, smem) != hipSuccess) return;
+            hipLaunchKernelGGL(kernel, grid, dim3(256), smem, st, s);
+        }
     } else if (threads == 128) {
         auto kernel = beam_step_kernel<CPL, LPR, U, GENERIC, 128>;
         if (vl_allow_lds(kernel, smem) != hipSuccess) return;
@@ -1694,20 +1718,26 @@ int dist_variant() {
 // The numbers after `false` are the sketch's lane shape for rows of that size (chunks per lane, lanes per row,
 // loads in flight), the wavefronts per SIMD asked for, the whole rows in flight in the sketch kernel (it fetches
 // few of them, so fewer in flight cost nothing and leave registers for another wavefront: 0.40 -> 0.36 ms per
-// launch at 384 columns) and, where given, the wavefronts per SIMD asked for in the kernels that run several
-// iterations per launch.  A sketch row has a quarter of the chunks, so a quarter of the lanes (or of the chunks
-// per lane) covers it.
+// launch at 384 columns), where given, the wavefronts per SIMD asked for in the kernels that run several
+// iterations per launch, and last the wavefronts per SIMD asked for in the kernel without the sketch
+// (beam_step_kernel_w; 0 = the compiler's own choice, which is seven at most: the step holds 106 scalar registers).
+// Eight wavefronts per SIMD - every workgroup slot a compute unit has - is what the launches that wait on memory
+// round trips rather than on bytes want, and the shapes that reach it without spilling a vector register ask for it
+// (measured: searches of 1M x 768 1.59 -> 1.69 M queries/s, the 1M x 128 build 4.4 -> 4.1 s; at 384 columns with
+// two instead of four whole rows in flight, third-loop launches 0.252 -> 0.217 ms, and the sketch kernel with one
+// load in flight 0.317 -> 0.295 ms on the first loop's).  A sketch row has a quarter of the chunks, so a quarter of
+// the lanes (or of the chunks per lane) covers it.
 int launch_step_by_dim(const StepArgs &s, bool aligned, int threads, size_t smem, hipStream_t st) {
     const int nchunks = s.nchunks;
     const int variant = dist_variant();
     if (!aligned || nchunks > 512) launch_step<1, 64, 1, true>(s, threads, smem, st);
-    else if (nchunks <= 16) launch_step<1, 16, 8, false, 1, 8, 4, 5, 8, 6>(s, threads, smem, st);
+    else if (nchunks <= 16) launch_step<1, 16, 8, false, 1, 8, 4, 5, 8, 6, 8>(s, threads, smem, st);
     else if (nchunks <= 32 && variant == 1) launch_step<1, 32, 8, false>(s, threads, smem, st);
-    else if (nchunks <= 32) launch_step<2, 16, 4, false, 1, 8, 4, 5, 4, 6>(s, threads, smem, st);
-    else if (nchunks <= 64) launch_step<1, 64, 8, false, 2, 8, 2, 5, 8, 6>(s, threads, smem, st);
-    else if (nchunks <= 96 && variant != 1) launch_step<3, 32, 4, false, 3, 8, 2, 6, 2>(s, threads, smem, st);
+    else if (nchunks <= 32) launch_step<2, 16, 4, false, 1, 8, 4, 5, 4, 6, 8>(s, threads, smem, st);
+    else if (nchunks <= 64) launch_step<1, 64, 8, false, 2, 8, 2, 5, 8, 6, 8>(s, threads, smem, st);
+    else if (nchunks <= 96 && variant != 1) launch_step<3, 32, 2, false, 3, 8, 1, 8, 1, 6, 8>(s, threads, smem, st);
     else if (nchunks <= 128) launch_step<2, 64, 8, false, 2, 16, 2, 6, 2>(s, threads, smem, st);
-    else if (nchunks <= 192) launch_step<3, 64, 2, false, 3, 16, 1, 8, 1, 6>(s, threads, smem, st);
+    else if (nchunks <= 192) launch_step<3, 64, 2, false, 3, 16, 1, 8, 1, 6, 8>(s, threads, smem, st);
     else if (nchunks <= 256) launch_step<4, 64, 4, false, 4, 16, 2, 5, 2>(s, threads, smem, st);
     else if (nchunks <= 320) launch_step<5, 64, 2, false, 3, 32, 2, 6, 1>(s, threads, smem, st);
     else if (nchunks <= 384) launch_step<6, 64, 2, false, 3, 32, 2, 6, 1>(s, threads, smem, st);
