@@ -374,10 +374,13 @@ def main():
                          "iteration, progress-check cadence, stop): a few hundred searches; off by default")
     ap.add_argument("--no-tuned", action="store_true", help="accepted for older command lines; the sweep is off by default")
     ap.add_argument("--search-runs", type=int, default=5, help="timed runs per search setting (the median is reported)")
-    ap.add_argument("--seed-dims", type=int, default=128,
+    ap.add_argument("--seed-dims", type=int, default=-1,
                     help="the dense seeding of the search leg ranks its 32,768 entry points by their first this many "
                          "columns (0 = all; seeds only have to land near the query); the all-column figure is reported "
-                         "beside it as search_full_rank_seeds")
+                         "beside it as search_full_rank_seeds.  Default: 64 for rows of 512 columns or more, else 128 "
+                         "(measured at 1M x 768, reference stop, recall@10 0.9994 throughout: 128 columns 1.69, "
+                         "96 1.74, 64 1.81, 48 1.82 M QPS, 32 columns 1.86 M at 0.9988; at 1M x 128 all 128 columns "
+                         "beat 64: 1.47 against 1.07 M QPS)")
     ap.add_argument("--queues", default="10,16,32,64,96,128,192,256",
                     help="search-queue lengths swept in this order (the sweep stops at the first that reaches recall@10 0.95)")
     ap.add_argument("--no-reference-seeding", action="store_true",
@@ -625,7 +628,8 @@ def main():
 
         # query-dependent seeds from dense MFMA tiles over 32,768 entry points (what reaches the recall target);
         # "batch" = the reference's stop (the whole batch runs until no row changed), bit-exact against the oracle
-        seed_dims = args.seed_dims if 0 < args.seed_dims < dim else None
+        wanted_dims = args.seed_dims if args.seed_dims >= 0 else (64 if dim >= 512 else 128)
+        seed_dims = wanted_dims if 0 < wanted_dims < dim else None
         if seed_dims is not None:
             result["search_full_rank_seeds"] = sweep_search("dense", "batch")
             ann.seed_dims, ann._entry = seed_dims, None
