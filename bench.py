@@ -381,6 +381,12 @@ def main():
                          "(measured at 1M x 768, reference stop, recall@10 0.9994 throughout: 128 columns 1.69, "
                          "96 1.74, 64 1.81, 48 1.82 M QPS, 32 columns 1.86 M at 0.9988; at 1M x 128 all 128 columns "
                          "beat 64: 1.47 against 1.07 M QPS)")
+    ap.add_argument("--seeds", type=int, default=-1,
+                    help="nearest entry points a query of the search leg starts from (0 = as many as its queue holds, "
+                         "16 at most).  Default: 4 for rows of 512 columns or more, else 0.  Measured with the "
+                         "reference stop at 1M x 768, recall@10 0.9994 throughout: 10 seeds 1.80, 8 1.84, 4 1.90, "
+                         "2 1.92, 1 seed 1.97 M QPS; at 1M x 128 (recall@10 0.83 either way) 10 seeds 1.47, 4 seeds "
+                         "1.05 M QPS: there a batch waits longer for its slowest query when it starts from fewer")
     ap.add_argument("--queues", default="10,16,32,64,96,128,192,256",
                     help="search-queue lengths swept in this order (the sweep stops at the first that reaches recall@10 0.95)")
     ap.add_argument("--no-reference-seeding", action="store_true",
@@ -628,13 +634,16 @@ def main():
 
         # query-dependent seeds from dense MFMA tiles over 32,768 entry points (what reaches the recall target);
         # "batch" = the reference's stop (the whole batch runs until no row changed), bit-exact against the oracle
+        wanted_seeds = args.seeds if args.seeds >= 0 else (4 if dim >= 512 else 0)
+        ann.dense_seeds = wanted_seeds if wanted_seeds > 0 else None
         wanted_dims = args.seed_dims if args.seed_dims >= 0 else (64 if dim >= 512 else 128)
         seed_dims = wanted_dims if 0 < wanted_dims < dim else None
         if seed_dims is not None:
             result["search_full_rank_seeds"] = sweep_search("dense", "batch")
             ann.seed_dims, ann._entry = seed_dims, None
         result["config"]["search_seeding"] = ("dense, 32768 entry points"
-                                              + (f" ranked by their first {seed_dims} columns" if seed_dims else ""))
+                                              + (f" ranked by their first {seed_dims} columns" if seed_dims else "")
+                                              + (f", {ann.dense_seeds} seeds per query" if ann.dense_seeds else ""))
         result["search"] = sweep_search("dense", "batch")
         # rows that are quiet stop expanding on their own (an addition; not bit-exact against the reference)
         result["search_per_query_stop"] = sweep_search("dense", "per_query")
@@ -649,10 +658,11 @@ def main():
         sr = step_roofline(profile_read(nv, reset=True, enable=0), dim, qdev.shape[0])
         (entry_ids, entry_vectors) = ann._entry_tables()
         ranked_by = qdev if entry_vectors.shape[1] == dim else qdev[:, :entry_vectors.shape[1]].contiguous()
-        knn_exact(ranked_by, entry_vectors, 16)
+        k_seed = min(ann.dense_seeds or 16, 16, qs)  # what dense_search_queue asks of the tiles
+        knn_exact(ranked_by, entry_vectors, k_seed)
         torch.cuda.synchronize()
         t0 = time.time()
-        knn_exact(ranked_by, entry_vectors, 16)
+        knn_exact(ranked_by, entry_vectors, k_seed)
         torch.cuda.synchronize()
         t_seed = time.time() - t0
         seed_flops = 2.0 * qdev.shape[0] * entry_vectors.shape[0] * entry_vectors.shape[1]

@@ -1096,6 +1096,24 @@ def test_dense_seeding_ranked_by_leading_columns():
     say(f"  recall@10 all columns {recall(a):.3f}, 16 of 64 columns {recall(b):.3f}")
     assert recall(b) > recall(a) - 0.05
 
+    # ANN(dense_seeds=k): a query starts from its k nearest entry points only - the oracle's loop from that very
+    # queue gives the same rows
+    few = ANN(dev(v), beams=full.beams, distances=full.distances, seeding="dense", entry_points=512, dense_seeds=3, **kw)
+    from vectorlink_gpu.ann import dense_search_queue
+    (entry_ids, entry_vectors) = few._entry_tables()
+    start = dense_search_queue(dev(v), dev(qv), few.configuration, entry_ids, entry_vectors, None, 3)
+    L = start.length
+    assert ((start.indices[:, :L] != M).sum(dim=1) == 3).all()
+    oq = orc.Queue(len(qv), L, start.indices.size(1))
+    oq.insert(host(start.indices)[:, :3], host(start.distances)[:, :3])
+    c = cfg(**kw)
+    t_want = orc.closest_vectors(qv, oq, v, host(full.beams), c, None)
+    got = few.search(dev(qv))
+    assert np.array_equal(host(got.indices)[:, :L], oq.indices[:, :L])
+    assert np.array_equal(bits(host(got.distances)[:, :L]), bits(oq.distances[:, :L]))
+    say(f"  3 seeds per query: {t_want} iterations, recall@10 {recall(got):.3f}")
+    assert recall(got) > recall(a) - 0.05
+
 
 def test_queues_beyond_64_kib_of_lds():
     """Degree 256 with a build queue of 512: 2048 candidates per iteration, a visit queue of 768 and a visited

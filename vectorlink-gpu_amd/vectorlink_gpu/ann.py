@@ -410,7 +410,8 @@ def entry_point_ids(vector_count: int, entry_points: int, device=DEVICE) -> Tens
 
 
 def dense_search_queue(vectors: Tensor, query_vectors: Tensor, config: Dict, entry_ids: Tensor,
-                       entry_vectors: Tensor, queue_size: Optional[int] = None) -> Queue:
+                       entry_vectors: Tensor, queue_size: Optional[int] = None,
+                       seeds: Optional[int] = None) -> Queue:
     # entry_vectors may hold only the first columns of the entry points (ANN.seed_dims): the seeds are
     # then ranked by that part of the dot product, which is enough to land near the query; the distances
     # that enter the queue are always the full ones.
@@ -425,7 +426,7 @@ def dense_search_queue(vectors: Tensor, query_vectors: Tensor, config: Dict, ent
     (batch_size, _) = query_vectors.size()
     extra_capacity = max(queue_size, config["parallel_visit_count"] * config["beam_size"])
     queue = Queue(batch_size, queue_size, queue_size + extra_capacity, device=vectors.device)
-    k = min(DENSE_SEEDS, entry_ids.size(0), queue_size)
+    k = min(seeds or DENSE_SEEDS, DENSE_SEEDS, entry_ids.size(0), queue_size)
     cols = entry_vectors.size(1)
     ranked_by = query_vectors if cols == query_vectors.size(1) else query_vectors[:, :cols].contiguous()
     (local, _) = knn_exact(ranked_by, entry_vectors, k, config.get("metric", "cosine"))
@@ -523,6 +524,7 @@ class ANN:
         concurrent_batches: int = 4,
         seed_dims: Optional[int] = None,
         sketch: bool = True,
+        dense_seeds: Optional[int] = None,
     ):
         """seeding / entry_points are additions: "circulant" seeds searches as the
         reference does; "dense" seeds them from the nearest of `entry_points`
@@ -532,6 +534,8 @@ class ANN:
         (kernels.optimize_graph) instead of keeping the first beam_size columns.
         seed_dims (with seeding="dense") ranks the entry points by their first seed_dims
         columns only - a cheaper pass that still lands near the query; None uses all.
+        dense_seeds (with seeding="dense") is the number of nearest entry points a query starts from
+        (None: as many as the search queue holds, 16 at most); the tile pass keeps shorter lists for fewer.
         concurrent_batches (an addition) is the number of batches of an optimisation loop
         that the build keeps in flight, each on its own stream and host thread; the
         graph does not depend on it.  metric is an addition too: "cosine" is the reference's distance; "l2" builds
@@ -546,6 +550,8 @@ class ANN:
         self.seeding = seeding
         self.entry_points = entry_points
         self.seed_dims = seed_dims
+        self.dense_seeds = dense_seeds
+        assert dense_seeds is None or dense_seeds >= 1
         assert seed_dims is None or (seed_dims > 0 and seed_dims % 4 == 0), "seed_dims must be a multiple of 4"
         self._entry = None
         self._queues = None
@@ -703,7 +709,7 @@ class ANN:
         if seeding == "dense":
             (entry_ids, entry_vectors) = self._entry_tables()
             search_queue = dense_search_queue(self.vectors, query, self.configuration, entry_ids, entry_vectors,
-                                              queue_size)
+                                              queue_size, self.dense_seeds)
         else:
             search_queue = initial_search_queue(self.vectors, query, self.configuration, queue_size)
         closest_vectors(query, search_queue, self.vectors, self.beams, self.configuration, None,
