@@ -21,6 +21,7 @@
 #include "rowsort.h"
 #include "dist_device.h"
 #include "sketch_device.h"
+#include <stddef.h>
 #include <stdlib.h>
 #include <atomic>
 #include <mutex>
@@ -2090,11 +2091,19 @@ int64_t beam_loop(const vl_beam_params *p, const BeamLayout &l, const float *que
             VL_LAUNCH_CHECK("beam merge kernel");
             if (prof) VL_HIP(hipEventRecord(ev[3 * r + 2], st));
         }
-        int changed = 0;
-        int state[2] = {0, 0};  // sketch_rows, error (neighbours in the control block)
-        VL_HIP(hipMemcpyAsync(&changed, &ctrl->changed[(t / R) & 63], sizeof(int), hipMemcpyDeviceToHost, st));
-        VL_HIP(hipMemcpyAsync(state, &ctrl->sketch_rows, sizeof(state), hipMemcpyDeviceToHost, st));
+        // one copy brings the ring of progress flags and the two words behind it (they are neighbours in the
+        // control block): this check's flag, the rows still using the sketch, the error flag
+        struct {
+            int changed[64];
+            int sketch_rows, error;
+        } seen_by_host;
+        static_assert(offsetof(BeamCtrl, error) - offsetof(BeamCtrl, changed) == 65 * sizeof(int) &&
+                          offsetof(BeamCtrl, sketch_rows) - offsetof(BeamCtrl, changed) == 64 * sizeof(int),
+                      "changed[64], sketch_rows, error follow each other");
+        VL_HIP(hipMemcpyAsync(&seen_by_host, &ctrl->changed[0], sizeof(seen_by_host), hipMemcpyDeviceToHost, st));
         VL_HIP(hipStreamSynchronize(st));
+        const int changed = seen_by_host.changed[(t / R) & 63];
+        const int state[2] = {seen_by_host.sketch_rows, seen_by_host.error};
         if (sketch_table) sketch_rows = state[0];
         if (state[1]) {
             vl_set_error("a row's visited list holds more ids than %lld iterations can have put there: the workspace "
