@@ -398,7 +398,7 @@ def main():
                          "seeding pass over 32,768 entry points); prints their figures as the JSON line")
     ap.add_argument("--cpu-rows", type=int, default=768)
     ap.add_argument("--loops", type=int, default=3, help="optimisation loops of the build (the reference's default is 3)")
-    ap.add_argument("--concurrent-batches", type=int, default=4,
+    ap.add_argument("--concurrent-batches", type=int, default=3,
                     help="batches of an optimisation loop kept in flight by the timed build (streams / host threads)")
     ap.add_argument("--no-sketch", action="store_true",
                     help="build without the 8-bit sketch of the vectors (every candidate row of the first loop is "
